@@ -1,0 +1,154 @@
+// C ABI of libfused_attn_gfx950.so: argument validation, launch geometry and the launch
+// itself.  Host counterpart of launch_attention_kernel (reference
+// include/fused_attn.cuh:860-894): picks the workgroup shape, sizes the dynamic LDS block,
+// builds the grid and launches on the caller's stream.
+#include "fused_attn_kernel.hpp"
+
+#include "../../include/fused_attn.h"
+
+#include <mutex>
+
+namespace {
+
+constexpr int kWaves = 4;       // wave64s per workgroup -> 256 query rows per workgroup
+constexpr int kKeyTile = 64;    // keys per LDS tile
+
+template <int H, bool HAS_MASK>
+hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
+    constexpr int lds = fa::lds_bytes<H, kWaves, kKeyTile>();
+    auto kernel = fa::fwd_kernel<H, kWaves, kKeyTile, HAS_MASK>;
+    // Dynamic LDS above 64 KiB has to be opted into once per kernel function.
+    if constexpr (lds > 64 * 1024) {
+        static std::once_flag once;
+        static hipError_t attr_status = hipSuccess;
+        std::call_once(once, [&] {
+            attr_status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        });
+        if (attr_status != hipSuccess) return attr_status;
+    }
+    const int grid = p.wgs_per_xcd * fa::kNumXcd;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kWaves * 64), lds, stream, p);
+    return hipGetLastError();
+}
+
+template <bool HAS_MASK>
+hipError_t dispatch(int64_t H, const fa::FwdParams& p, hipStream_t stream) {
+    switch (H) {
+        case 16: return launch<16, HAS_MASK>(p, stream);
+        case 32: return launch<32, HAS_MASK>(p, stream);
+        case 64: return launch<64, HAS_MASK>(p, stream);
+        case 128: return launch<128, HAS_MASK>(p, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+int validate(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,
+             int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h, int64_t stride_l,
+             fa::FwdParams* p, float scale) {
+    if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return FA_ERR_NULL_POINTER;
+    if (!fa_fwd_query(H)) return FA_ERR_BAD_HEAD_DIM;
+    if (B < 1 || R < 1 || L < 1) return FA_ERR_BAD_SHAPE;
+    if (stride_l < H || stride_h < 0 || stride_b < 0) return FA_ERR_BAD_STRIDE;
+    if ((stride_l % 8) != 0 || (stride_h % 8) != 0 || (stride_b % 8) != 0) return FA_ERR_BAD_STRIDE;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return FA_ERR_MISALIGNED;
+    if (mask != nullptr && (reinterpret_cast<uintptr_t>(mask) & 1u) != 0) return FA_ERR_MISALIGNED;
+    constexpr int64_t kMaxInt = 0x7fffffff;
+    if (L > kMaxInt - 4096 || B > kMaxInt || R > kMaxInt) return FA_ERR_TOO_LARGE;
+    const int64_t bq = kWaves * 64;
+    const int64_t n_qtiles = (L + bq - 1) / bq;
+    const int64_t total = B * R * n_qtiles;
+    if (total > kMaxInt - 8 || B * R > kMaxInt) return FA_ERR_TOO_LARGE;
+    constexpr int64_t kMaxElems = (int64_t)1 << 62;
+    if (L > kMaxElems / stride_l || (stride_h > 0 && R > kMaxElems / stride_h) ||
+        (stride_b > 0 && B > kMaxElems / stride_b))
+        return FA_ERR_TOO_LARGE;
+
+    p->q = static_cast<const _Float16*>(q);
+    p->k = static_cast<const _Float16*>(k);
+    p->v = static_cast<const _Float16*>(v);
+    p->mask = static_cast<const _Float16*>(mask);
+    p->o = static_cast<_Float16*>(out);
+    p->stride_b = stride_b;
+    p->stride_h = stride_h;
+    p->stride_l = stride_l;
+    p->B = (int)B;
+    p->R = (int)R;
+    p->L = (int)L;
+    p->n_qtiles = (int)n_qtiles;
+    p->total_wgs = (int)total;
+    p->wgs_per_xcd = (int)((total + fa::kNumXcd - 1) / fa::kNumXcd);
+    p->scale_log2e = scale * 1.4426950408889634f;
+    return FA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fa_fwd_query(int64_t H) { return (H == 16 || H == 32 || H == 64 || H == 128) ? 1 : 0; }
+
+const char* fa_strerror(int status) {
+    switch (status) {
+        case FA_OK: return "success";
+        case FA_ERR_NULL_POINTER: return "fa_fwd: q, k, v and out must be non-null device pointers";
+        case FA_ERR_BAD_HEAD_DIM: return "fa_fwd: head_dim must be 16, 32, 64 or 128";
+        case FA_ERR_BAD_SHAPE: return "fa_fwd: B, R and L must be at least 1";
+        case FA_ERR_BAD_STRIDE:
+            return "fa_fwd: strides must be non-negative multiples of 8 elements and stride_l >= head_dim";
+        case FA_ERR_MISALIGNED: return "fa_fwd: q, k, v and out must be 16-byte aligned";
+        case FA_ERR_TOO_LARGE: return "fa_fwd: problem size exceeds the supported index range";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
+    return "fa_fwd: unknown status";
+}
+
+int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,
+           int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h, int64_t stride_l,
+           float scale, void* stream) {
+    fa::FwdParams p;
+    const int rc = validate(q, k, v, mask, out, B, R, L, H, stride_b, stride_h, stride_l, &p, scale);
+    if (rc != FA_OK) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const hipError_t e = mask != nullptr ? dispatch<true>(H, p, s) : dispatch<false>(H, p, s);
+    return static_cast<int>(e);
+}
+
+int fa_fwd_timed(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,
+                 int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h,
+                 int64_t stride_l, float scale, void* stream, int iters, float* ms_per_launch) {
+    if (ms_per_launch == nullptr) return FA_ERR_NULL_POINTER;
+    if (iters < 1) return FA_ERR_BAD_SHAPE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipEventCreate(&e0);
+    if (e != hipSuccess) return static_cast<int>(e);
+    e = hipEventCreate(&e1);
+    if (e != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return static_cast<int>(e);
+    }
+    int rc = FA_OK;
+    e = hipEventRecord(e0, s);
+    if (e != hipSuccess) rc = static_cast<int>(e);
+    for (int i = 0; i < iters && rc == FA_OK; ++i)
+        rc = fa_fwd(q, k, v, mask, out, B, R, L, H, stride_b, stride_h, stride_l, scale, stream);
+    if (rc == FA_OK) {
+        e = hipEventRecord(e1, s);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+        if (e == hipSuccess)
+            *ms_per_launch = ms / (float)iters;
+        else
+            rc = static_cast<int>(e);
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return rc;
+}
+
+}  // extern "C"

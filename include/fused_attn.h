@@ -1,0 +1,85 @@
+/*
+ * C ABI of the gfx950 fused multi-head attention forward library
+ * (libfused_attn_gfx950.so).  Plain pointers and sizes only: no torch types, no HIP
+ * types in the signatures, so the same entry points can be bound from C++, ctypes or
+ * any FFI.
+ *
+ * All tensors are IEEE fp16 in device memory.  q, k, v and out share one addressing
+ * rule, given in ELEMENTS:
+ *     element(b, h, l, d) = base + b*stride_b + h*stride_h + l*stride_l + d      (d < H)
+ * The reference layout [B, L, R*H] (reference src/fused_attn_extention.cu:24-27,50-52;
+ * head h = columns [h*H, (h+1)*H), reference include/fused_attn.cuh:683-690) is
+ *     stride_b = L*R*H, stride_h = H, stride_l = R*H,
+ * and a [B, R, L, H] tensor is stride_b = R*L*H, stride_h = L*H, stride_l = H.
+ * Strides must be multiples of 8 elements and the base pointers 16-byte aligned.
+ *
+ * Return value of every int function: 0 = success, < 0 = invalid argument (FA_ERR_*),
+ * > 0 = a hipError_t raised by the runtime.  Nothing here ever calls exit().
+ */
+#ifndef FUSED_ATTN_H_
+#define FUSED_ATTN_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FA_OK 0
+#define FA_ERR_NULL_POINTER (-1)
+#define FA_ERR_BAD_HEAD_DIM (-2)
+#define FA_ERR_BAD_SHAPE (-3)
+#define FA_ERR_BAD_STRIDE (-4)
+#define FA_ERR_MISALIGNED (-5)
+#define FA_ERR_TOO_LARGE (-6)
+
+/*
+ * out = softmax(q k^T * scale [+ mask]) v for every (batch, head), non-causal.
+ *
+ * Replaces launch_attention_kernel<head_dim, chunk_size>(batch_size, seq_len,
+ * num_features, queries, keys, values, mask, output, syncronize)
+ * (reference include/fused_attn.cuh:860-894) together with the kernel it launches
+ * (reference include/fused_attn.cuh:605-858).  Differences a caller can see:
+ *   - head_dim is a run-time argument (16, 32, 64 or 128), there is no chunk_size:
+ *     the key tile is an internal choice and L need not be a multiple of anything;
+ *   - the launch goes to `stream` (a hipStream_t, NULL = the null stream) and the
+ *     call returns without synchronising;
+ *   - `mask` (nullable) is an additive fp16 [B, L, L] tensor shared by all heads and is
+ *     applied to every key, not only to the first chunk.  Rows whose keys are all -inf
+ *     produce zeros.
+ * B, R, L >= 1.  L*stride_l, R*stride_h and B*stride_b must stay below 2^62 elements.
+ */
+int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* out,
+           int64_t B, int64_t R, int64_t L, int64_t H,
+           int64_t stride_b, int64_t stride_h, int64_t stride_l,
+           float scale, void* stream);
+
+/*
+ * 1 if fa_fwd accepts this head_dim, else 0.  Counterpart of the compile-time
+ * (head_dim, chunk_size) dispatch table (reference src/fused_attn_extention.cu:72-111).
+ */
+int fa_fwd_query(int64_t H);
+
+/*
+ * Human-readable text for a status returned by fa_fwd.  Replaces the print-and-exit
+ * macros CHECK_CUDA_ERROR / CHECK_LAST_CUDA_ERROR (reference include/fused_attn.cuh:17-42).
+ * The returned pointer is static storage.
+ */
+const char* fa_strerror(int status);
+
+/*
+ * Timed replay for benchmarks: launches fa_fwd `iters` times back to back on `stream`,
+ * bracketed by HIP events recorded on that same stream, waits, and writes the average
+ * milliseconds per launch to *ms_per_launch.  Counterpart of the timing loop in
+ * reference tests/benchmark_fused_attn.py:36-42 (wall clock around 128 launches).
+ */
+int fa_fwd_timed(const void* q, const void* k, const void* v, const void* mask, void* out,
+                 int64_t B, int64_t R, int64_t L, int64_t H,
+                 int64_t stride_b, int64_t stride_h, int64_t stride_l,
+                 float scale, void* stream, int iters, float* ms_per_launch);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FUSED_ATTN_H_ */
