@@ -1,0 +1,141 @@
+"""Benchmark of the fused attention forward on one MI355X.
+
+One step = one forward pass (softmax(Q K^T / sqrt(H)) V for every batch and head) over one
+synthetic batch resident in HBM.  Prints one JSON line: whole-job TFLOP/s with
+flop = 4*B*R*L^2*H, the MFMA roofline of the kernel (average launch duration from HIP events
+recorded on the launch stream inside the kernel library) and, beside it, the naive float32 CPU
+evaluation of the same workload timed on the host cores over a bounded sample of (batch, head)
+pairs.  Counterpart of the reference's benchmark (reference tests/benchmark_fused_attn.py:8-45),
+which prints wall-clock milliseconds of 128 naive and 128 fused launches.
+
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5a|c5b|readme]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+if REPO not in sys.path:
+    sys.path.insert(0, REPO)
+
+PEAK_TFLOPS_FP16 = 2500.0   # MI355X dense fp16 MFMA, published
+
+
+def cpu_baseline(w, q, k, v, gpu_out, budget_s):
+    """Naive float32 attention on the host cores for a bounded sample of (batch, head) pairs.
+
+    The checker (oracle/) is used here as the timed CPU baseline and to report the error of the
+    GPU result on the sampled pairs; it never produces anything the benchmark's `value` uses.
+    """
+    import torch
+
+    from oracle import attention_per_head
+
+    cores = torch.get_num_threads()
+    pairs_all = [(b, h) for b in range(w.B) for h in range(w.R)]
+    t0 = time.perf_counter()
+    attention_per_head(q, k, v, w.H, heads=pairs_all[:1])         # warm-up, also sizes the sample
+    per_pair = time.perf_counter() - t0
+    n = max(1, min(len(pairs_all), int(budget_s / max(per_pair, 1e-6))))
+    stride = max(1, len(pairs_all) // n)
+    pairs = pairs_all[::stride][:n]
+    t0 = time.perf_counter()
+    ref = attention_per_head(q, k, v, w.H, heads=pairs)
+    dt = time.perf_counter() - t0
+    flop = 4.0 * len(pairs) * w.L * w.L * w.H
+    sel = ~torch.isnan(ref)
+    err = (gpu_out.float().cpu()[sel] - ref[sel]).abs().max().item()
+    return {
+        "value": flop / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": "%d of %d (batch, head) pairs of %s, torch float32 per-head loop, %.2f s"
+                  % (len(pairs), len(pairs_all), w.name, dt),
+        "ms_per_step_extrapolated": dt / len(pairs) * len(pairs_all) * 1e3,
+        "gpu_max_abs_err_on_sample": err,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c3")
+    ap.add_argument("--cpu-budget-s", type=float, default=15.0,
+                    help="seconds of host time for the CPU baseline sample (0 disables it)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the forward has no multi-GPU path "
+                 "(every (batch, head) pair is independent); run with --gpus 1")
+
+    import torch
+
+    import fused_attn
+    from fused_attention_amd import capi, workloads
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    capi.load_library()     # fail loudly if the kernel library is not built
+    w = workloads.WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    q, k, v = workloads.make_inputs(w)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    chunk = min(128, w.H * 2)
+
+    for _ in range(args.warmup):
+        out = fused_attn.attention_forward(w.H, chunk, qd, kd, vd)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = fused_attn.attention_forward(w.H, chunk, qd, kd, vd)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+
+    # Kernel duration: HIP events on the launch stream around back-to-back launches.
+    kernel_ms = capi.forward_timed(qd, kd, vd, w.H, out, iters=args.steps)
+
+    flop = workloads.flops(w)
+    value = flop / (ms_per_step * 1e-3) / 1e12
+    achieved = flop / (kernel_ms * 1e-3) / 1e12
+    line = {
+        "metric": "fused attn fwd TFLOP/s (4*B*R*L^2*H)",
+        "value": value,
+        "unit": "TFLOP/s",
+        "pct_of_fp16_mfma_peak": 100.0 * value / PEAK_TFLOPS_FP16,
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: B=%d R=%d L=%d H=%d non-causal, fp16 N(0,%g) seeded on the host, "
+                        "fed as [B, L, R*H]" % (w.name, w.B, w.R, w.L, w.H, w.q_std),
+            "flop_per_step": flop,
+            "bytes_per_step": workloads.io_bytes(w),
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": PEAK_TFLOPS_FP16,
+            "unit": "TFLOP/s",
+            "frac": achieved / PEAK_TFLOPS_FP16,
+            "traffic": None,
+            "kernel_ms": kernel_ms,
+        },
+    }
+    if args.cpu_budget_s > 0:
+        line["cpu_baseline"] = cpu_baseline(w, q, k, v, out, args.cpu_budget_s)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

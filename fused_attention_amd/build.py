@@ -75,7 +75,7 @@ def build_torch_binding():
         cmd += ["-I" + inc]
     cmd += [os.path.join(CSRC, "fused_attn_extention.cpp"), "-o", ext_path(),
             "-L" + PKG_DIR, "-lfused_attn_gfx950",
-            "-L" + torch_lib, "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_python",
+            "-L" + torch_lib, "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip", "-ltorch_python",
             "-Wl,-rpath,$ORIGIN/fused_attention_amd", "-Wl,-rpath," + torch_lib,
             "-Wl,--no-as-needed"]
     _run(cmd)

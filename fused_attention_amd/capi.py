@@ -1,0 +1,120 @@
+"""ctypes view of libfused_attn_gfx950.so (the C ABI declared in include/fused_attn.h).
+
+The functions here only marshal pointers, sizes and strides; all checking of those values is
+done by the library and reported through its status codes.
+"""
+import ctypes
+import math
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libfused_attn_gfx950.so")
+
+# every symbol include/fused_attn.h declares
+EXPORTS = ("fa_fwd", "fa_fwd_query", "fa_strerror", "fa_fwd_timed")
+
+_lib = None
+
+
+class FusedAttnError(RuntimeError):
+    """A non-zero status from the kernel library."""
+
+    def __init__(self, status, text):
+        super().__init__("%s (status %d)" % (text, status))
+        self.status = status
+
+
+def load_library():
+    """Loads the kernel library once.  Raises OSError if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise OSError(
+            "%s is missing: build it with `python -m fused_attention_amd.build` "
+            "(there is no fallback implementation)" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    i64, vp, f32 = ctypes.c_int64, ctypes.c_void_p, ctypes.c_float
+    fwd_args = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, f32, vp]
+    lib.fa_fwd.argtypes = fwd_args
+    lib.fa_fwd.restype = ctypes.c_int
+    lib.fa_fwd_timed.argtypes = fwd_args + [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+    lib.fa_fwd_timed.restype = ctypes.c_int
+    lib.fa_fwd_query.argtypes = [i64]
+    lib.fa_fwd_query.restype = ctypes.c_int
+    lib.fa_strerror.argtypes = [ctypes.c_int]
+    lib.fa_strerror.restype = ctypes.c_char_p
+    _lib = lib
+    return lib
+
+
+def strerror(status):
+    return load_library().fa_strerror(int(status)).decode()
+
+
+def _check(status):
+    if status != 0:
+        raise FusedAttnError(status, strerror(status))
+
+
+def fwd_raw(q_ptr, k_ptr, v_ptr, mask_ptr, out_ptr, B, R, L, H, stride_b, stride_h, stride_l,
+            scale, stream=0):
+    """fa_fwd on raw device addresses (ints).  Returns the status code without raising."""
+    return load_library().fa_fwd(q_ptr, k_ptr, v_ptr, mask_ptr or None, out_ptr, B, R, L, H,
+                                 stride_b, stride_h, stride_l, scale, stream or None)
+
+
+def _layout(q, head_dim, layout):
+    if layout == "blf":      # [B, L, R*H]: the reference layout
+        B, L, F = q.shape
+        R = F // head_dim
+        return B, R, L, L * F, head_dim, F
+    if layout == "bhld":     # [B, R, L, H]
+        B, R, L, H = q.shape
+        return B, R, L, R * L * H, L * H, H
+    raise ValueError("layout must be 'blf' or 'bhld'")
+
+
+def _current_stream(q):
+    import torch
+
+    return torch.cuda.current_stream(q.device).cuda_stream
+
+
+def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None):
+    """Runs fa_fwd on torch GPU tensors (fp16, contiguous) on torch's current stream.
+
+    layout 'blf' takes [B, L, R*head_dim] tensors, 'bhld' takes [B, R, L, head_dim] tensors.
+    Returns `out` (allocated like q when not given).
+    """
+    import torch
+
+    B, R, L, sb, sh, sl = _layout(q, head_dim, layout)
+    if out is None:
+        out = torch.empty_like(q)
+    if scale is None:
+        scale = 1.0 / math.sqrt(head_dim)
+    with torch.cuda.device(q.device):
+        status = fwd_raw(q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                         mask.data_ptr() if mask is not None else 0, out.data_ptr(),
+                         B, R, L, head_dim, sb, sh, sl, scale, _current_stream(q))
+    _check(status)
+    return out
+
+
+def forward_timed(q, k, v, head_dim, out, iters, mask=None, layout="blf", scale=None):
+    """Average milliseconds per launch over `iters` back-to-back launches (HIP events on the
+    launch stream, measured inside the library)."""
+    import torch
+
+    B, R, L, sb, sh, sl = _layout(q, head_dim, layout)
+    if scale is None:
+        scale = 1.0 / math.sqrt(head_dim)
+    ms = ctypes.c_float(0.0)
+    with torch.cuda.device(q.device):
+        status = load_library().fa_fwd_timed(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr() if mask is not None else None,
+            out.data_ptr(), B, R, L, head_dim, sb, sh, sl, scale, _current_stream(q) or None,
+            int(iters), ctypes.byref(ms))
+    _check(status)
+    return float(ms.value)

@@ -1,0 +1,113 @@
+// PyTorch-ROCm binding of the gfx950 fused attention forward: Python module `fused_attn`.
+//
+// Host-only C++ (compiled by g++, no device code): it validates the tensors, allocates the
+// output and hands raw device pointers plus torch's current HIP stream to the C ABI of
+// libfused_attn_gfx950.so.  It keeps the entry point of the reference binding
+// (reference src/fused_attn_extention.cu:15-22 and :119-129): same module name, same function
+// name, same argument names, order and default.
+//
+// Contract kept from the reference (src/fused_attn_extention.cu:24-64):
+//   queries, keys, values : fp16, on the GPU, contiguous, 3-D [batch, seq_len, num_features],
+//                           equal shapes, num_features % head_dim == 0
+//   mask (optional)       : fp16, on the GPU, contiguous, 3-D
+//   head_dim, chunk_size  : powers of two, 16 <= head_dim <= 128, 16 <= chunk_size <= 128,
+//                           chunk_size <= 2 * head_dim, not (chunk_size 16 with head_dim 128)
+//   returns               : new fp16 [batch, seq_len, num_features] tensor
+// Deliberate differences:
+//   - seq_len need not be a multiple of chunk_size (the reference rejects it at :63); the key
+//     tile is chosen by the kernel library and chunk_size is only validated;
+//   - the mask must be [batch, seq_len, seq_len] and is applied to every key;
+//   - the output lives on the device of `queries` and the launch goes to torch's current
+//     stream (the reference uses the default device and the legacy default stream);
+//   - every rejected argument raises with a message, and a launch failure raises instead of
+//     terminating the process (reference include/fused_attn.cuh:17-42 calls std::exit).
+#include <torch/extension.h>
+
+// PyTorch-ROCm presents its HIP devices under the device type "cuda"; these are the guard and
+// stream accessors that understand that.
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+
+#include <cmath>
+
+#include "fused_attn.h"
+
+namespace {
+
+void check_qkv(const torch::Tensor& t, const char* name) {
+    TORCH_CHECK(t.dtype() == torch::kFloat16, name, " must be float16, got ", t.dtype());
+    TORCH_CHECK(t.device().type() == torch::kCUDA, name, " must be a GPU tensor, got device ",
+                t.device());
+    TORCH_CHECK(t.dim() == 3, name, " must be 3-D [batch, seq_len, num_features], got ", t.dim(),
+                " dimensions");
+    TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+}
+
+bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
+
+torch::Tensor attention_forward(int64_t head_dim, int64_t chunk_size, torch::Tensor queries,
+                                torch::Tensor keys, torch::Tensor values,
+                                std::optional<torch::Tensor> mask) {
+    TORCH_CHECK(is_pow2(head_dim) && 16 <= head_dim && head_dim <= 128,
+                "head_dim must be a power of two in [16, 128], got ", head_dim);
+    TORCH_CHECK(is_pow2(chunk_size) && 16 <= chunk_size && chunk_size <= 128,
+                "chunk_size must be a power of two in [16, 128], got ", chunk_size);
+    TORCH_CHECK(chunk_size <= 2 * head_dim, "chunk_size must not exceed 2 * head_dim, got chunk_size ",
+                chunk_size, " with head_dim ", head_dim);
+    TORCH_CHECK(!(chunk_size == 16 && head_dim == 128),
+                "chunk_size 16 with head_dim 128 is not a supported combination");
+    TORCH_CHECK(fa_fwd_query(head_dim) == 1, "head_dim ", head_dim,
+                " is not supported by the kernel library");
+
+    check_qkv(queries, "queries");
+    check_qkv(keys, "keys");
+    check_qkv(values, "values");
+
+    const int64_t batch_size = queries.size(0);
+    const int64_t seq_len = queries.size(1);
+    const int64_t num_features = queries.size(2);
+    TORCH_CHECK(keys.sizes() == queries.sizes(), "keys must have the shape of queries ",
+                queries.sizes(), ", got ", keys.sizes());
+    TORCH_CHECK(values.sizes() == queries.sizes(), "values must have the shape of queries ",
+                queries.sizes(), ", got ", values.sizes());
+    TORCH_CHECK(keys.device() == queries.device() && values.device() == queries.device(),
+                "queries, keys and values must be on the same device");
+    TORCH_CHECK(batch_size >= 1 && seq_len >= 1 && num_features >= 1,
+                "queries must not have an empty dimension, got ", queries.sizes());
+    TORCH_CHECK(num_features % head_dim == 0, "num_features (", num_features,
+                ") must be a multiple of head_dim (", head_dim, ")");
+
+    const void* mask_ptr = nullptr;
+    if (mask.has_value()) {
+        const torch::Tensor& m = *mask;
+        TORCH_CHECK(m.dtype() == torch::kFloat16, "mask must be float16, got ", m.dtype());
+        TORCH_CHECK(m.device() == queries.device(), "mask must be on the device of queries");
+        TORCH_CHECK(m.dim() == 3 && m.is_contiguous(), "mask must be a contiguous 3-D tensor");
+        TORCH_CHECK(m.size(0) == batch_size && m.size(1) == seq_len && m.size(2) == seq_len,
+                    "mask must have shape [batch, seq_len, seq_len] = [", batch_size, ", ", seq_len,
+                    ", ", seq_len, "], got ", m.sizes());
+        mask_ptr = m.data_ptr<at::Half>();
+    }
+
+    const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(queries.device());
+    torch::Tensor output = torch::empty_like(queries);
+    const int64_t num_heads = num_features / head_dim;
+    const float scale = 1.0f / std::sqrt(static_cast<float>(head_dim));
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(queries.device().index()).stream();
+
+    const int status = fa_fwd(queries.data_ptr<at::Half>(), keys.data_ptr<at::Half>(),
+                              values.data_ptr<at::Half>(), mask_ptr, output.data_ptr<at::Half>(),
+                              batch_size, num_heads, seq_len, head_dim,
+                              /*stride_b=*/seq_len * num_features, /*stride_h=*/head_dim,
+                              /*stride_l=*/num_features, scale, static_cast<void*>(stream));
+    TORCH_CHECK(status == FA_OK, "fused attention launch failed: ", fa_strerror(status));
+    return output;
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    m.def("attention_forward", &attention_forward, py::arg("head_dim"), py::arg("chunk_size"),
+          py::arg("queries"), py::arg("keys"), py::arg("values"),
+          py::arg("mask") = std::optional<torch::Tensor>(), "Fused multihead attention");
+}

@@ -1,0 +1,254 @@
+"""GPU parity of the fused attention forward against the CPU oracle.
+
+Mirrors the reference's test strategy (reference tests/test_fused_attn.py:12-67: one case per
+legal (head_dim, chunk_size), B=1, two heads, two chunks, seed 179, N(0,1) inputs) and adds what
+the reference never tested: batch > 1, more than two heads, many key tiles, sequence lengths that
+are not tile multiples, large-magnitude scores, closed-form answers and the strided C-ABI entry.
+
+Tolerance: max |fused.float() - oracle_fp32| <= 5e-3 and every output finite.  The reference's
+own bound (rtol = atol = 1e-2, tests/test_fused_attn.py:30) is checked as well in the drop-in cases.
+"""
+import math
+
+import pytest
+import torch
+
+from fused_attention_amd import capi, workloads
+from oracle import attention, attention_per_head
+
+pytestmark = pytest.mark.gpu
+
+TOL = 5e-3
+
+
+def _max_err(got, want):
+    got = got.float().cpu()
+    assert torch.isfinite(got).all(), "non-finite output"
+    return (got - want).abs().max().item()
+
+
+def _rand(shape, seed, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * std).to(torch.float16)
+
+
+# ---- the reference's 12 (head_dim, chunk_size) cases, through the torch binding ---------------
+
+LEGAL = [(16, 16), (16, 32), (32, 16), (32, 32), (32, 64), (64, 16), (64, 32), (64, 64), (64, 128),
+         (128, 32), (128, 64), (128, 128)]
+
+
+@pytest.mark.parametrize("head_dim,chunk_size", LEGAL)
+def test_simple(gpu, head_dim, chunk_size):
+    import fused_attn
+
+    torch.random.manual_seed(179)
+    batch_size, num_heads, num_chunks = 1, 2, 2
+    num_features = num_heads * head_dim
+    sequence_len = num_chunks * chunk_size
+    queries, keys, values = (torch.randn(batch_size, sequence_len, num_features).half() for _ in range(3))
+
+    expected = attention(queries, keys, values, head_dim)
+    actual = fused_attn.attention_forward(head_dim, chunk_size, queries.to(gpu), keys.to(gpu), values.to(gpu))
+
+    assert actual.shape == queries.shape and actual.dtype == torch.float16 and actual.device.type == "cuda"
+    torch.testing.assert_close(actual.float().cpu(), expected, rtol=0.01, atol=0.01)
+    assert _max_err(actual, expected) <= TOL
+
+
+# ---- benchmark configurations -------------------------------------------------------------------
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c5a", "c5b"])
+def test_config_full_tensor(gpu, name):
+    import fused_attn
+
+    w = workloads.WORKLOADS[name]
+    q, k, v = workloads.make_inputs(w)
+    want = attention_per_head(q, k, v, w.H)
+    got = fused_attn.attention_forward(w.H, 64, q.to(gpu), k.to(gpu), v.to(gpu))
+    assert _max_err(got, want) <= TOL
+    if name.startswith("c5"):
+        # the stress inputs really do reach large scores
+        s = (q[0, :, :w.H].float() @ k[0, :, :w.H].float().T) / math.sqrt(w.H)
+        assert s.abs().max() > 20
+
+
+def test_config_c3_headline(gpu):
+    import fused_attn
+
+    w = workloads.WORKLOADS["c3"]
+    q, k, v = workloads.make_inputs(w)
+    got = fused_attn.attention_forward(w.H, 64, q.to(gpu), k.to(gpu), v.to(gpu)).float().cpu()
+    assert torch.isfinite(got).all()
+    # every row of a third of the (batch, head) pairs, spread over batches and heads
+    pairs = [(b, h) for b in range(w.B) for h in range(w.R) if (b * w.R + h) % 3 == 0]
+    want = attention_per_head(q, k, v, w.H, heads=pairs)
+    sel = ~torch.isnan(want)
+    assert (got[sel] - want[sel]).abs().max().item() <= TOL
+    # size-independent property on the whole tensor: a convex combination stays inside the range of V
+    vmax = v.float().view(w.B, w.L, w.R, w.H).abs().amax(dim=1, keepdim=True).expand(w.B, w.L, w.R, w.H)
+    assert (got.view(w.B, w.L, w.R, w.H).abs() <= vmax + 1e-3).all()
+
+
+def test_config_c4_sampled_heads(gpu):
+    import fused_attn
+
+    w = workloads.WORKLOADS["c4"]
+    q, k, v = workloads.make_inputs(w)
+    got = fused_attn.attention_forward(w.H, 128, q.to(gpu), k.to(gpu), v.to(gpu)).float().cpu()
+    assert torch.isfinite(got).all()
+    pairs = [(0, 0), (0, 13), (0, 31)]       # first, middle and last head; all 16384 rows of each
+    want = attention_per_head(q, k, v, w.H, heads=pairs)
+    sel = ~torch.isnan(want)
+    assert (got[sel] - want[sel]).abs().max().item() <= TOL
+
+
+# ---- shapes the reference never exercised ---------------------------------------------------------
+
+@pytest.mark.parametrize("B,R,L,H", [
+    (1, 1, 1, 64), (1, 1, 2, 16), (2, 3, 31, 32), (1, 2, 33, 64), (3, 5, 63, 64), (2, 2, 65, 128),
+    (1, 3, 255, 64), (2, 2, 257, 64), (1, 2, 511, 32), (2, 7, 300, 16), (1, 1, 1025, 128), (1, 40, 129, 128),
+])
+def test_ragged_and_odd_shapes(gpu, B, R, L, H):
+    q, k, v = (_rand((B, L, R * H), 1000 + L + i) for i in range(3))
+    want = attention(q, k, v, H)
+    out = torch.full_like(q, float("nan"), device=gpu)
+    capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, out=out)
+    assert _max_err(out, want) <= TOL
+
+
+def test_native_bhld_layout_matches_packed_layout(gpu):
+    B, R, L, H = 2, 3, 200, 64
+    q, k, v = (_rand((B, L, R * H), 2000 + i).to(gpu) for i in range(3))
+    packed = capi.forward(q, k, v, H)
+    qb, kb, vb = (workloads.to_bhld(t, H) for t in (q, k, v))
+    native = capi.forward(qb, kb, vb, H, layout="bhld")
+    assert torch.equal(native.transpose(1, 2).reshape(B, L, R * H), packed)
+
+
+def test_runs_on_the_current_stream_and_is_deterministic(gpu):
+    import fused_attn
+
+    w = workloads.WORKLOADS["c1"]
+    q, k, v = (t.to(gpu) for t in workloads.make_inputs(w))
+    first = fused_attn.attention_forward(w.H, 64, q, k, v)
+    side = torch.cuda.Stream(device=gpu)
+    side.wait_stream(torch.cuda.current_stream(gpu))
+    with torch.cuda.stream(side):
+        second = fused_attn.attention_forward(w.H, 64, q, k, v)
+    side.synchronize()
+    assert torch.equal(first, second)
+
+
+# ---- closed forms (no oracle involved) ---------------------------------------------------------------
+
+@pytest.mark.parametrize("L", [1000, 3073])
+def test_zero_queries_return_the_mean_over_the_true_keys(gpu, L):
+    # Catches tail-padding leakage: padded keys would enter the mean.
+    B, R, H = 1, 2, 64
+    k, v = _rand((B, L, R * H), 3000, 3.0), _rand((B, L, R * H), 3001)
+    out = capi.forward(torch.zeros_like(k).to(gpu), k.to(gpu), v.to(gpu), H)
+    want = v.double().mean(dim=1, keepdim=True).float().expand(B, L, R * H)
+    assert _max_err(out, want) <= 1e-3
+
+
+def test_constant_values_are_returned(gpu):
+    B, R, L, H = 2, 2, 777, 64
+    q, k = _rand((B, L, R * H), 3100, 3.0), _rand((B, L, R * H), 3101, 3.0)
+    v = torch.full((B, L, R * H), 1.5, dtype=torch.float16)
+    out = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H)
+    assert _max_err(out, v.float()) <= 1e-3
+
+
+def test_one_hot_retrieval_with_huge_scores(gpu):
+    # Orthogonal keys (scaled Hadamard-like sign codes); query i points at key pi(i) with score 90+.
+    H, L = 64, 64
+    had = torch.tensor([[1.0]])
+    while had.shape[0] < H:
+        had = torch.cat([torch.cat([had, had], 1), torch.cat([had, -had], 1)], 0)
+    k = (had * 3.0).to(torch.float16).view(1, L, H)
+    perm = torch.randperm(L, generator=torch.Generator().manual_seed(7))
+    q = (k[0, perm] * 1.5).contiguous().view(1, L, H)    # matching score 4.5*3*64/8 = 108, others 0
+    v = _rand((1, L, H), 3200)
+    out = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H)
+    assert _max_err(out, v[0, perm].float().view(1, L, H)) <= 1e-3
+
+
+def test_shift_and_duplication_invariance(gpu):
+    B, R, L, H = 1, 2, 320, 64
+    q, k, v = (_rand((B, L, R * H), 3300 + i) for i in range(3))
+    base = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H).float().cpu()
+    # a constant added to every key shifts each score row by q.delta/sqrt(H): the running max moves
+    # by a large amount while the weights stay the same
+    delta = torch.zeros(1, 1, R * H, dtype=torch.float16)
+    delta[..., ::2] = 4.0
+    shifted = capi.forward(q.to(gpu), (k + delta).to(gpu), v.to(gpu), H).float().cpu()
+    assert (shifted - base).abs().max().item() <= 3e-3
+    dup = capi.forward(q.repeat(1, 2, 1).to(gpu), k.repeat(1, 2, 1).to(gpu), v.repeat(1, 2, 1).to(gpu), H)
+    assert (dup.float().cpu()[:, :L] - base).abs().max().item() <= 2e-3
+
+
+def test_heads_and_batches_are_independent_bitwise(gpu):
+    B, R, L, H = 2, 3, 130, 64
+    q, k, v = (_rand((B, L, R * H), 3400 + i) for i in range(3))
+    base = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H).cpu()
+    q2, k2, v2 = q.clone(), k.clone(), v.clone()
+    for t in (q2, k2, v2):
+        t[0, :, H:2 * H] = t[0, :, H:2 * H] * 0.5 + 1.0
+    out = capi.forward(q2.to(gpu), k2.to(gpu), v2.to(gpu), H).cpu()
+    assert torch.equal(out[1], base[1])
+    assert torch.equal(out[0, :, :H], base[0, :, :H]) and torch.equal(out[0, :, 2 * H:], base[0, :, 2 * H:])
+    assert not torch.equal(out[0, :, H:2 * H], base[0, :, H:2 * H])
+
+
+# ---- additive mask ---------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("L,H", [(64, 64), (200, 32), (300, 128)])
+def test_additive_mask_on_every_key_tile(gpu, L, H):
+    import fused_attn
+
+    B, R = 2, 2
+    q, k, v = (_rand((B, L, R * H), 3500 + i) for i in range(3))
+    g = torch.Generator().manual_seed(3510)
+    mask = torch.where(torch.rand(B, L, L, generator=g) < 0.3, float("-inf"), 0.0)
+    mask = (mask + torch.randn(B, L, L, generator=g) * 0.5).to(torch.float16)
+    mask[:, :, 0] = 0                                   # keep at least one key per row
+    want = attention(q, k, v, H, mask=mask)
+    got = fused_attn.attention_forward(H, 32, q.to(gpu), k.to(gpu), v.to(gpu), mask.to(gpu))
+    assert _max_err(got, want) <= TOL
+
+
+def test_fully_masked_rows_give_zeros_not_nan(gpu):
+    B, R, L, H = 1, 2, 100, 64
+    q, k, v = (_rand((B, L, R * H), 3600 + i) for i in range(3))
+    mask = torch.zeros(B, L, L, dtype=torch.float16)
+    mask[0, 5] = float("-inf")
+    mask[0, 77] = float("-inf")
+    out = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, mask=mask.to(gpu)).float().cpu()
+    assert torch.isfinite(out).all()
+    assert (out[0, 5] == 0).all() and (out[0, 77] == 0).all()
+    want = attention(q, k, v, H)
+    keep = [i for i in range(L) if i not in (5, 77)]
+    assert (out[0, keep] - want[0, keep]).abs().max().item() <= TOL
+
+
+# ---- argument rejection that needs device tensors ---------------------------------------------------
+
+def test_binding_rejections_on_device_tensors(gpu):
+    import fused_attn
+
+    x = torch.zeros(2, 64, 128, dtype=torch.float16, device=gpu)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        fused_attn.attention_forward(64, 64, x.transpose(0, 1), x, x)
+    with pytest.raises(RuntimeError, match="3-D"):
+        fused_attn.attention_forward(64, 64, x[0], x, x)
+    with pytest.raises(RuntimeError, match="shape of queries"):
+        fused_attn.attention_forward(64, 64, x, x[:, :32].contiguous(), x)
+    with pytest.raises(RuntimeError, match="multiple of head_dim"):
+        fused_attn.attention_forward(128, 64, x[:, :, :64].contiguous(), x[:, :, :64].contiguous(),
+                                     x[:, :, :64].contiguous())
+    with pytest.raises(RuntimeError, match="mask must have shape"):
+        fused_attn.attention_forward(64, 64, x, x, x, torch.zeros(2, 64, 32, dtype=torch.float16, device=gpu))
+    # a sequence length that is not a multiple of chunk_size is accepted (the reference rejects it)
+    y = torch.zeros(1, 50, 64, dtype=torch.float16, device=gpu)
+    assert fused_attn.attention_forward(64, 64, y, y, y).shape == y.shape

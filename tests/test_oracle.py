@@ -1,0 +1,168 @@
+"""Pins the CPU oracle (oracle/) before anything is compared against it.  No GPU needed.
+
+Each check is chosen so that a plausible mistake in the restatement fails it: a wrong head split
+(columns of head h), a wrong scale (1/H instead of 1/sqrt(H)), softmax over the wrong axis, a
+transposed operand, a mask applied to the wrong axis.
+"""
+import ctypes
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention, attention_f64, attention_per_head
+
+ORACLE_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle")
+
+
+def _rand(shape, seed, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * std).to(torch.float16)
+
+
+def _c_oracle():
+    path = os.path.join(ORACLE_DIR, "libattention_ref.so")
+    if not os.path.exists(path):
+        pytest.skip("oracle/libattention_ref.so not built (make -C oracle)")
+    lib = ctypes.CDLL(path)
+    fp = ctypes.POINTER(ctypes.c_float)
+    lib.attention_ref_f64.argtypes = [fp, fp, fp, fp, ctypes.POINTER(ctypes.c_double)] + [ctypes.c_int64] * 4
+    lib.attention_ref_f64.restype = ctypes.c_int
+    return lib
+
+
+def _run_c(q, k, v, head_dim, mask=None):
+    lib = _c_oracle()
+    B, L, F = q.shape
+    arrs = [np.ascontiguousarray(t.float().numpy()) for t in (q, k, v)]
+    fp = ctypes.POINTER(ctypes.c_float)
+    m = np.ascontiguousarray(mask.float().numpy()) if mask is not None else None
+    out = np.empty((B, L, F), dtype=np.float64)
+    rc = lib.attention_ref_f64(*[a.ctypes.data_as(fp) for a in arrs],
+                               m.ctypes.data_as(fp) if m is not None else None,
+                               out.ctypes.data_as(ctypes.POINTER(ctypes.c_double)), B, L, F // head_dim, head_dim)
+    assert rc == 0
+    return out
+
+
+@pytest.mark.parametrize("B,R,L,H", [(1, 2, 32, 16), (2, 3, 77, 32), (1, 4, 256, 64), (1, 2, 130, 128)])
+def test_against_plain_c_and_numpy_f64(B, R, L, H):
+    q, k, v = (_rand((B, L, R * H), 10 + i) for i in range(3))
+    got = attention(q, k, v, H).double().numpy()
+    ref_c = _run_c(q, k, v, H)
+    ref_np = attention_f64(q.float().numpy(), k.float().numpy(), v.float().numpy(), H)
+    np.testing.assert_allclose(ref_np, ref_c, rtol=0, atol=1e-12)
+    np.testing.assert_allclose(got, ref_c, rtol=0, atol=2e-6)
+
+
+@pytest.mark.parametrize("B,R,L,H", [(2, 4, 100, 64), (1, 3, 513, 32)])
+def test_against_library_sdpa(B, R, L, H):
+    q, k, v = (_rand((B, L, R * H), 20 + i) for i in range(3))
+
+    def split(x):
+        return x.float().view(B, L, R, H).transpose(1, 2)
+
+    lib = torch.nn.functional.scaled_dot_product_attention(split(q), split(k), split(v))
+    lib = lib.transpose(1, 2).reshape(B, L, R * H)
+    torch.testing.assert_close(attention(q, k, v, H), lib, rtol=0, atol=2e-6)
+
+
+def test_per_head_form_is_the_same_arithmetic():
+    B, R, L, H = 2, 3, 150, 64
+    q, k, v = (_rand((B, L, R * H), 30 + i) for i in range(3))
+    torch.testing.assert_close(attention_per_head(q, k, v, H), attention(q, k, v, H), rtol=0, atol=1e-6)
+    part = attention_per_head(q, k, v, H, heads=[(1, 2)])
+    assert torch.isnan(part[0]).all() and torch.isnan(part[1, :, : 2 * H]).all()
+    torch.testing.assert_close(part[1, :, 2 * H:], attention(q, k, v, H)[1, :, 2 * H:], rtol=0, atol=1e-6)
+
+
+def test_head_h_is_columns_hH_to_hH_plus_H():
+    # V of head h is the constant h + 1: whatever the weights, head h's output columns equal h + 1.
+    B, R, L, H = 1, 4, 19, 16
+    q, k = _rand((B, L, R * H), 40), _rand((B, L, R * H), 41)
+    v = torch.arange(1, R + 1, dtype=torch.float16).repeat_interleave(H).expand(B, L, R * H).contiguous()
+    out = attention(q, k, v, H)
+    want = torch.arange(1, R + 1, dtype=torch.float32).repeat_interleave(H).expand(B, L, R * H)
+    torch.testing.assert_close(out, want, rtol=0, atol=1e-5)
+
+
+def test_heads_and_batches_do_not_mix():
+    B, R, L, H = 2, 3, 40, 32
+    q, k, v = (_rand((B, L, R * H), 50 + i) for i in range(3))
+    base = attention(q, k, v, H)
+    q2, k2, v2 = q.clone(), k.clone(), v.clone()
+    for t in (q2, k2, v2):
+        t[0, :, H:2 * H] += 1.0   # disturb head 1 of batch 0 only
+    out = attention(q2, k2, v2, H)
+    assert torch.equal(out[0, :, :H], base[0, :, :H]) and torch.equal(out[0, :, 2 * H:], base[0, :, 2 * H:])
+    assert torch.equal(out[1], base[1])
+    assert not torch.equal(out[0, :, H:2 * H], base[0, :, H:2 * H])
+
+
+@pytest.mark.parametrize("H", [16, 64])
+def test_scale_is_one_over_sqrt_head_dim(H):
+    # Two keys; q.k0 = a*b, q.k1 = 0  =>  weight on key 0 is sigmoid(a*b/sqrt(H)).
+    a, b = 3.0, 2.0
+    q = torch.zeros(1, 2, H, dtype=torch.float16)
+    k = torch.zeros(1, 2, H, dtype=torch.float16)
+    v = torch.zeros(1, 2, H, dtype=torch.float16)
+    q[0, :, 0] = a
+    k[0, 0, 0] = b
+    v[0, 0, :] = 1.0
+    v[0, 1, :] = -1.0
+    w = 1.0 / (1.0 + math.exp(-a * b / math.sqrt(H)))
+    out = attention(q, k, v, H)
+    torch.testing.assert_close(out, torch.full_like(out, 2 * w - 1), rtol=0, atol=1e-6)
+
+
+def test_zero_queries_give_the_column_mean_of_values():
+    B, R, L, H = 2, 2, 333, 32
+    k, v = _rand((B, L, R * H), 60), _rand((B, L, R * H), 61)
+    out = attention(torch.zeros_like(k), k, v, H)
+    want = v.float().mean(dim=1, keepdim=True).expand_as(out)
+    torch.testing.assert_close(out, want, rtol=0, atol=1e-5)
+
+
+def test_single_key_returns_values():
+    q, k, v = (_rand((3, 1, 128), 70 + i) for i in range(3))
+    assert torch.equal(attention(q, k, v, 64), v.float())
+
+
+def test_one_hot_retrieval():
+    # Keys are scaled basis vectors, query i is a large multiple of key pi(i): row i returns V[pi(i)].
+    H = L = 32
+    k = (torch.eye(L) * 8.0).to(torch.float16).view(1, L, H)
+    perm = torch.randperm(L, generator=torch.Generator().manual_seed(5))
+    q = (k[0, perm] * 4.0).view(1, L, H)            # score of the matching key: 256/sqrt(32) = 45
+    v = _rand((1, L, H), 80)
+    out = attention(q, k, v, H)
+    torch.testing.assert_close(out[0], v[0, perm].float(), rtol=0, atol=1e-6)
+
+
+def test_invariances_permutation_shift_duplication():
+    B, R, L, H = 1, 2, 96, 32
+    q, k, v = (_rand((B, L, R * H), 90 + i) for i in range(3))
+    base = attention(q, k, v, H)
+    perm = torch.randperm(L, generator=torch.Generator().manual_seed(6))
+    torch.testing.assert_close(attention(q, k[:, perm], v[:, perm], H), base, rtol=0, atol=2e-6)
+    # adding one vector to every key shifts each score row by a constant
+    delta = _rand((1, 1, R * H), 93)
+    torch.testing.assert_close(attention(q, (k.float() + delta.float()), v, H), base, rtol=0, atol=2e-5)
+    # concatenating (K, V) with itself leaves the weighted mean unchanged
+    dup = attention(q.repeat(1, 2, 1), k.repeat(1, 2, 1), v.repeat(1, 2, 1), H)
+    torch.testing.assert_close(dup[:, :L], base, rtol=0, atol=2e-6)
+
+
+def test_additive_mask_removes_keys():
+    B, R, L, H = 2, 2, 50, 32
+    q, k, v = (_rand((B, L, R * H), 100 + i) for i in range(3))
+    keep = 17
+    mask = torch.zeros(B, L, L, dtype=torch.float16)
+    mask[:, :, keep:] = float("-inf")
+    masked = attention(q, k, v, H, mask=mask)
+    # the first `keep` query rows of the masked call see exactly the shortened problem
+    short = attention(*(t[:, :keep].contiguous() for t in (q, k, v)), H)
+    torch.testing.assert_close(masked[:, :keep], short, rtol=0, atol=2e-6)
+    np.testing.assert_allclose(masked.double().numpy(), _run_c(q, k, v, H, mask=mask), rtol=0, atol=2e-6)
