@@ -147,13 +147,56 @@ struct TileLoader {
     }
 };
 
+// Largest partial row sum (16 terms) the fast path of the online softmax accepts.
+constexpr float kTrip = 16384.f;
+
+// p = exp2(s * c + mc) for the 2 x 16 scores of a sub-tile, rounded to fp16 pairs (round toward
+// zero), and the per-lane sums of the rounded values.  The sums are taken over the rounded
+// probabilities that enter the second product, so numerator and denominator see the same rounding.
+__device__ __forceinline__ void exp_pack_sum(const floatx16 (&s)[2], float c, const float (&mc)[2],
+                                             uint32_t (&pk)[2][8], float (&ts)[2]) {
+    const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+        float acc = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nb][r], c, mc[nb]));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nb][r + 1], c, mc[nb]));
+            const uint32_t pp = pack_rtz(p0, p1);
+            pk[nb][r >> 1] = pp;
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, pp), ones, acc, false);
+        }
+        ts[nb] = acc;
+    }
+}
+
+// O^T[.][nb] *= alpha, in place.  Written as one instruction per register with the register tied
+// as input and output, so that the rarely taken rescale does not make the compiler keep a second
+// copy of the accumulators (and copy them on the common path).  The leading wait covers the
+// matrix-core results the multiplies read.
+template <int DB>
+__device__ __forceinline__ void scale_accumulators(floatx16 (&o)[DB][2], int nb, float alpha) {
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float e = o[db][nb][r];
+            asm volatile("v_mul_f32 %0, %1, %0" : "+v"(e) : "v"(alpha));
+            o[db][nb][r] = e;
+        }
+    }
+}
+
 // Per-wave state: Q^T as B operands, O^T accumulators, online-softmax (m, l).
 template <int H>
 struct WaveState {
     using G = Geometry<H>;
     half8 q[2][G::KS];
     floatx16 o[G::DB][2];
-    float m[2];   // running row max of the raw (unscaled) scores, identical in lanes l and l^32
+    float m[2];   // reference row maximum of the raw (unscaled) scores, identical in lanes l and l^32
+    float mc[2];  // -m * c, the additive term of the exponent; +inf while no reference exists yet
     float l[2];   // running sum of exp over the keys this lane has seen (half of each tile)
 };
 
@@ -222,44 +265,42 @@ __device__ __forceinline__ void process_subtile(WaveState<H>& st, const _Float16
     }
 
     // ---- online softmax ------------------------------------------------------------------
+    // Fast path: exponentiate against the reference maximum of the rows seen so far, without
+    // looking at this sub-tile's maximum.  Any reference works as long as numerator and
+    // denominator share it; it only has to keep exp2 inside the fp16 range.  Each lane checks
+    // that with its own partial row sum: 16 non-negative terms whose sum is <= kTrip are each
+    // <= kTrip, and anything that overflowed (inf) or was computed from an undefined reference
+    // (NaN) fails the comparison.  Only then the wave takes the slow path, which brings the
+    // reference up to the true running maximum and rescales O and l.
     uint32_t pk[2][8];
+    float ts[2];
+    exp_pack_sum(s, c, st.mc, pk, ts);
+    const bool ok = (ts[0] <= kTrip) & (ts[1] <= kTrip);
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!ok) != 0, 0)) {
+        float mcu[2];
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-        float mx = fmax2(s[nb][0], s[nb][1]);
+        for (int nb = 0; nb < 2; ++nb) {
+            float mx = fmax2(s[nb][0], s[nb][1]);
 #pragma unroll
-        for (int r = 2; r < 16; r += 2) mx = fmax2(mx, fmax2(s[nb][r], s[nb][r + 1]));
-        mx = pair_max(mx);
-        const float m_old = st.m[nb];
-        const float m_new = fmax2(m_old, mx);
-        // Rescale only when some row of this block saw a new maximum (wave-uniform branch).
-        if (__builtin_amdgcn_ballot_w64(m_new > m_old) != 0) {
-            // m_new == -inf can only happen while every key so far was masked by an additive
-            // -inf mask; keep alpha finite (the accumulators are still zero then).
-            const float alpha = (m_new == -__builtin_inff())
-                                    ? 1.f
-                                    : __builtin_amdgcn_exp2f((m_old - m_new) * c);
+            for (int r = 2; r < 16; r += 2) mx = fmax2(mx, fmax2(s[nb][r], s[nb][r + 1]));
+            mx = pair_max(mx);
+            const float m_old = st.m[nb];
+            const float m_new = fmax2(m_old, mx);
+            // m_new == -inf: every key so far carried a -inf additive mask.  Nothing has been
+            // accumulated yet, this sub-tile contributes zeros, and the stored reference stays
+            // undefined (+inf) so that the next sub-tile comes back here.
+            const bool empty = m_new == -__builtin_inff();
+            const float alpha = empty ? 1.f : __builtin_amdgcn_exp2f((m_old - m_new) * c);
             st.l[nb] *= alpha;
-#pragma unroll
-            for (int db = 0; db < G::DB; ++db)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) st.o[db][nb][r] *= alpha;
+            scale_accumulators<G::DB>(st.o, nb, alpha);
             st.m[nb] = m_new;
+            st.mc[nb] = empty ? __builtin_inff() : -m_new * c;
+            mcu[nb] = empty ? 0.f : -m_new * c;
         }
-        const float mc = (m_new == -__builtin_inff()) ? 0.f : -m_new * c;
-        float lsum = st.l[nb];
-#pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nb][r], c, mc));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nb][r + 1], c, mc));
-            const uint32_t pp = pack_rtz(p0, p1);
-            pk[nb][r >> 1] = pp;
-            // The row sum is taken over the f16-rounded probabilities that enter the second
-            // product, so numerator and denominator see the same rounding.
-            const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
-            lsum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, pp), ones, lsum, false);
-        }
-        st.l[nb] = lsum;
+        exp_pack_sum(s, c, mcu, pk, ts);
     }
+    st.l[0] += ts[0];
+    st.l[1] += ts[1];
 
     // ---- O^T += V_sub^T * P^T ------------------------------------------------------------
     // Transpose read: inside each group of 16 lanes, lane j receives, for i = 0..3, element
@@ -344,6 +385,7 @@ __global__ __launch_bounds__(NW * 64, (H <= 64 ? 2 : 1)) void fwd_kernel(const F
             st.q[nb][kk] = __builtin_bit_cast(half8, w);
         }
         st.m[nb] = -__builtin_inff();
+        st.mc[nb] = __builtin_inff();
         st.l[nb] = 0.f;
 #pragma unroll
         for (int db = 0; db < G::DB; ++db)
@@ -367,34 +409,34 @@ __global__ __launch_bounds__(NW * 64, (H <= 64 ? 2 : 1)) void fwd_kernel(const F
     loader.store(ks_base, vs_base, tid);
     __syncthreads();
 
-    for (int t = 0; t < ntiles; ++t) {
+    // Full tiles: one straight path per iteration.  The ragged last tile, if any, is peeled off so
+    // that its masking code does not share a loop (and register assignment) with the hot path.
+    const int nfull = L / BK;
+    for (int t = 0; t < nfull; ++t) {
         const int buf = t & 1;
         const _Float16* ks = ks_base + buf * BK * G::KSTR;
         const _Float16* vs = vs_base + buf * BK * G::VSTR;
         const bool has_next = t + 1 < ntiles;
         if (has_next) loader.load(kbase, vbase, p.stride_l, (t + 1) * BK, L, tid);
-
-        const int key0 = t * BK;
-        if (key0 + BK <= L) {
 #pragma unroll
-            for (int sub = 0; sub < NSUB; ++sub)
-                process_subtile<H, false, HAS_MASK>(st, ks, vs, sub, 32, c, lane, mask_row0, mask_row1,
-                                                    key0 + sub * 32, L);
-        } else {
-#pragma unroll
-            for (int sub = 0; sub < NSUB; ++sub) {
-                const int nvalid = L - key0 - sub * 32;
-                if (nvalid > 0)
-                    process_subtile<H, true, HAS_MASK>(st, ks, vs, sub, nvalid, c, lane, mask_row0,
-                                                       mask_row1, key0 + sub * 32, L);
-            }
-        }
-
-        if (has_next) {
-            const int nbuf = buf ^ 1;
-            loader.store(ks_base + nbuf * BK * G::KSTR, vs_base + nbuf * BK * G::VSTR, tid);
-        }
+        for (int sub = 0; sub < NSUB; ++sub)
+            process_subtile<H, false, HAS_MASK>(st, ks, vs, sub, 32, c, lane, mask_row0, mask_row1,
+                                                t * BK + sub * 32, L);
+        if (has_next) loader.store(ks_base + (buf ^ 1) * BK * G::KSTR, vs_base + (buf ^ 1) * BK * G::VSTR, tid);
         __syncthreads();
+    }
+    if (nfull < ntiles) {
+        const int buf = nfull & 1;
+        const _Float16* ks = ks_base + buf * BK * G::KSTR;
+        const _Float16* vs = vs_base + buf * BK * G::VSTR;
+        const int key0 = nfull * BK;
+#pragma unroll
+        for (int sub = 0; sub < NSUB; ++sub) {
+            const int nvalid = L - key0 - sub * 32;
+            if (nvalid > 0)
+                process_subtile<H, true, HAS_MASK>(st, ks, vs, sub, nvalid, c, lane, mask_row0, mask_row1,
+                                                   key0 + sub * 32, L);
+        }
     }
 
     // ---- epilogue: O = O^T / l, f16, 8-byte stores ------------------------------------------
