@@ -10,11 +10,21 @@
 
 namespace {
 
-constexpr int kWaves = 4;       // wave64s per workgroup -> 256 query rows per workgroup
-constexpr int kKeyTile = 64;    // keys per LDS tile
+constexpr int kKeyTile = 64;     // keys per LDS tile
+constexpr int kNumCu = 256;      // compute units of one MI355X
 
-template <int H, bool HAS_MASK>
+// Wave64s per workgroup (64 query rows each).  Eight waves share one K/V stream between twice
+// as many queries, which pays once there are enough workgroups to give every compute unit two of
+// them; head_dim 128 needs the whole register file of a SIMD for one wave, so it stays at four.
+int pick_waves(int64_t B, int64_t R, int64_t L, int64_t H) {
+    if (H > 64) return 4;
+    const int64_t wgs8 = B * R * ((L + 511) / 512);
+    return wgs8 >= 2 * kNumCu ? 8 : 4;
+}
+
+template <int H, int NW, bool HAS_MASK>
 hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
+    constexpr int kWaves = NW;
     constexpr int lds = fa::lds_bytes<H, kWaves, kKeyTile>();
     auto kernel = fa::fwd_kernel<H, kWaves, kKeyTile, HAS_MASK>;
     // Dynamic LDS above 64 KiB has to be opted into once per kernel function.
@@ -33,12 +43,12 @@ hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
 }
 
 template <bool HAS_MASK>
-hipError_t dispatch(int64_t H, const fa::FwdParams& p, hipStream_t stream) {
+hipError_t dispatch(int64_t H, int waves, const fa::FwdParams& p, hipStream_t stream) {
     switch (H) {
-        case 16: return launch<16, HAS_MASK>(p, stream);
-        case 32: return launch<32, HAS_MASK>(p, stream);
-        case 64: return launch<64, HAS_MASK>(p, stream);
-        case 128: return launch<128, HAS_MASK>(p, stream);
+        case 16: return waves == 8 ? launch<16, 8, HAS_MASK>(p, stream) : launch<16, 4, HAS_MASK>(p, stream);
+        case 32: return waves == 8 ? launch<32, 8, HAS_MASK>(p, stream) : launch<32, 4, HAS_MASK>(p, stream);
+        case 64: return waves == 8 ? launch<64, 8, HAS_MASK>(p, stream) : launch<64, 4, HAS_MASK>(p, stream);
+        case 128: return launch<128, 4, HAS_MASK>(p, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -47,7 +57,7 @@ bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u
 
 int validate(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,
              int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h, int64_t stride_l,
-             fa::FwdParams* p, float scale) {
+             fa::FwdParams* p, float scale, int* waves) {
     if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return FA_ERR_NULL_POINTER;
     if (!fa_fwd_query(H)) return FA_ERR_BAD_HEAD_DIM;
     if (B < 1 || R < 1 || L < 1) return FA_ERR_BAD_SHAPE;
@@ -57,7 +67,8 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     if (mask != nullptr && (reinterpret_cast<uintptr_t>(mask) & 1u) != 0) return FA_ERR_MISALIGNED;
     constexpr int64_t kMaxInt = 0x7fffffff;
     if (L > kMaxInt - 4096 || B > kMaxInt || R > kMaxInt) return FA_ERR_TOO_LARGE;
-    const int64_t bq = kWaves * 64;
+    *waves = pick_waves(B, R, L, H);
+    const int64_t bq = *waves * 64;
     const int64_t n_qtiles = (L + bq - 1) / bq;
     const int64_t total = B * R * n_qtiles;
     if (total > kMaxInt - 8 || B * R > kMaxInt) return FA_ERR_TOO_LARGE;
@@ -110,10 +121,11 @@ int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* 
            int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h, int64_t stride_l,
            float scale, void* stream) {
     fa::FwdParams p;
-    const int rc = validate(q, k, v, mask, out, B, R, L, H, stride_b, stride_h, stride_l, &p, scale);
+    int waves = 4;
+    const int rc = validate(q, k, v, mask, out, B, R, L, H, stride_b, stride_h, stride_l, &p, scale, &waves);
     if (rc != FA_OK) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const hipError_t e = mask != nullptr ? dispatch<true>(H, p, s) : dispatch<false>(H, p, s);
+    const hipError_t e = mask != nullptr ? dispatch<true>(H, waves, p, s) : dispatch<false>(H, waves, p, s);
     return static_cast<int>(e);
 }
 

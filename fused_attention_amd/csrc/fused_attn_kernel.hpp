@@ -102,7 +102,8 @@ __device__ __forceinline__ uint32_t pack_rtz(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
 }
 
-// Streams one K/V tile from global memory into registers, and from registers into LDS.
+// Streams K/V tiles from global memory into registers, and from registers into LDS.  K and V are
+// handled separately because the pipelined loop keeps K one tile ahead of V.
 template <int H, int NW, int BK>
 struct TileLoader {
     using G = Geometry<H>;
@@ -110,41 +111,39 @@ struct TileLoader {
     static constexpr int NCHUNK = BK * CPR;
     static constexpr int NT = NW * 64;
     static constexpr int NP = (NCHUNK + NT - 1) / NT;       // chunks per thread
+    static constexpr bool EXACT = NCHUNK % NT == 0;
     u32x4 kreg[NP];
     u32x4 vreg[NP];
 
-    __device__ __forceinline__ void load(const _Float16* kbase, const _Float16* vbase,
-                                         int64_t stride_l, int key0, int L, int tid) {
+    static __device__ __forceinline__ void load(u32x4 (&reg)[NP], const _Float16* base, int64_t stride_l,
+                                                int key0, int L, int tid) {
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
             const int idx = tid + i * NT;
-            const int row = idx / CPR;
-            const int chunk = idx % CPR;
-            const int key = key0 + row;
-            u32x4 kk = {0u, 0u, 0u, 0u};
-            u32x4 vv = {0u, 0u, 0u, 0u};
-            if ((NCHUNK % NT == 0 || idx < NCHUNK) && key < L) {
-                const int64_t off = (int64_t)key * stride_l + chunk * 8;
-                kk = *reinterpret_cast<const u32x4*>(kbase + off);
-                vv = *reinterpret_cast<const u32x4*>(vbase + off);
-            }
-            kreg[i] = kk;
-            vreg[i] = vv;
+            const int key = key0 + idx / CPR;
+            u32x4 x = {0u, 0u, 0u, 0u};   // rows past the end of the sequence read as zeros
+            if ((EXACT || idx < NCHUNK) && key < L)
+                x = *reinterpret_cast<const u32x4*>(base + (int64_t)key * stride_l + (idx % CPR) * 8);
+            reg[i] = x;
         }
     }
-
-    __device__ __forceinline__ void store(_Float16* ks, _Float16* vs, int tid) const {
+    template <int STR>
+    static __device__ __forceinline__ void store(const u32x4 (&reg)[NP], _Float16* dst, int tid) {
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
             const int idx = tid + i * NT;
-            const int row = idx / CPR;
-            const int chunk = idx % CPR;
-            if (NCHUNK % NT == 0 || idx < NCHUNK) {
-                *reinterpret_cast<u32x4*>(ks + row * G::KSTR + chunk * 8) = kreg[i];
-                *reinterpret_cast<u32x4*>(vs + row * G::VSTR + chunk * 8) = vreg[i];
-            }
+            if (EXACT || idx < NCHUNK)
+                *reinterpret_cast<u32x4*>(dst + (idx / CPR) * STR + (idx % CPR) * 8) = reg[i];
         }
     }
+    __device__ __forceinline__ void load_k(const _Float16* kbase, int64_t sl, int key0, int L, int tid) {
+        load(kreg, kbase, sl, key0, L, tid);
+    }
+    __device__ __forceinline__ void load_v(const _Float16* vbase, int64_t sl, int key0, int L, int tid) {
+        load(vreg, vbase, sl, key0, L, tid);
+    }
+    __device__ __forceinline__ void store_k(_Float16* ks, int tid) const { store<G::KSTR>(kreg, ks, tid); }
+    __device__ __forceinline__ void store_v(_Float16* vs, int tid) const { store<G::VSTR>(vreg, vs, tid); }
 };
 
 // Largest partial row sum (16 terms) the fast path of the online softmax accepts.
@@ -200,121 +199,53 @@ struct WaveState {
     float l[2];   // running sum of exp over the keys this lane has seen (half of each tile)
 };
 
-// Processes 32 keys (one sub-tile) for the wave's 64 queries.
-//   ks/vs : LDS tile base for the current buffer
-//   sub   : sub-tile index inside the tile
-//   nvalid: number of valid keys in this sub-tile (only read when MASKED)
-template <int H, bool MASKED, bool HAS_MASK>
-__device__ __forceinline__ void process_subtile(WaveState<H>& st, const _Float16* ks,
-                                                const _Float16* vs, int sub, int nvalid,
-                                                float c, int lane,
-                                                const _Float16* mask_row0, const _Float16* mask_row1,
-                                                int key_base, int L) {
-    using G = Geometry<H>;
-    const int g = lane >> 5;
-    const int ln = lane & 31;
+// LDS address of this lane's K row for sub-tile `sub` of a tile: A operand of S^T = K_sub * Q^T.
+template <int H>
+__device__ __forceinline__ const _Float16* k_operand_ptr(const _Float16* ks, int sub, int lane) {
+    return ks + (sub * 32 + (lane & 31)) * Geometry<H>::KSTR + 8 * (lane >> 5);
+}
 
-    // ---- S^T = K_sub * Q^T -------------------------------------------------------------
-    floatx16 s[2];
+// LDS address this lane hands to the transpose reads of sub-tile `sub`.  Inside each group of 16
+// lanes, lane j receives, for i = 0..3, element (j % 4) of the 8-byte row fetched by lane
+// 4 i + j / 4.  With lane s of a group pointing at V[key0 + s / 4][d0 + 4 (s % 4) ...], lane j ends
+// up with V[key0 + i][d0 + j], i = 0..3: four consecutive keys of one head-dim column.
+template <int H>
+__device__ __forceinline__ const _Float16* v_operand_ptr(const _Float16* vs, int sub, int lane) {
+    const int s16 = lane & 15;
+    return vs + (sub * 32 + 4 * (lane >> 5) + (s16 >> 2)) * Geometry<H>::VSTR + 16 * ((lane >> 4) & 1) +
+           4 * (s16 & 3);
+}
+
+// S^T = K_sub * Q^T for 32 keys and the wave's 2 x 32 queries.
+template <int H>
+__device__ __forceinline__ void qk_mfma(floatx16 (&s)[2], const half8 (&q)[2][Geometry<H>::KS],
+                                        const _Float16* krow) {
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[nb][r] = 0.f;
-
-    const _Float16* krow = ks + (sub * 32 + ln) * G::KSTR + 8 * g;
 #pragma unroll
-    for (int kk = 0; kk < G::KS; ++kk) {
+    for (int kk = 0; kk < Geometry<H>::KS; ++kk) {
         const half8 a = *reinterpret_cast<const half8*>(krow + kk * 16);
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb)
-            s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, st.q[nb][kk], s[nb], 0, 0, 0);
+            s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, q[nb][kk], s[nb], 0, 0, 0);
     }
+}
 
-    // ---- optional additive mask (log2 domain is applied later, so pre-divide by c) -------
-    if constexpr (HAS_MASK) {
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-            const _Float16* mrow = nb == 0 ? mask_row0 : mask_row1;
-            if (mrow != nullptr) {
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    const int key = key_base + 8 * r4 + 4 * g;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if (key + j < L) {
-                            // The mask is added to the scaled score; S holds raw scores, so the
-                            // mask is brought to raw units: (s*scale + mask) = scale*(s + mask/scale).
-                            s[nb][4 * r4 + j] += (float)mrow[key + j] * (1.4426950408889634f / c);
-                        }
-                    }
-                }
-            }
-        }
-    }
-
-    // ---- tail masking --------------------------------------------------------------------
-    if constexpr (MASKED) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int key = 8 * (r >> 2) + 4 * g + (r & 3);
-            if (key >= nvalid) {
-                s[0][r] = -__builtin_inff();
-                s[1][r] = -__builtin_inff();
-            }
-        }
-    }
-
-    // ---- online softmax ------------------------------------------------------------------
-    // Fast path: exponentiate against the reference maximum of the rows seen so far, without
-    // looking at this sub-tile's maximum.  Any reference works as long as numerator and
-    // denominator share it; it only has to keep exp2 inside the fp16 range.  Each lane checks
-    // that with its own partial row sum: 16 non-negative terms whose sum is <= kTrip are each
-    // <= kTrip, and anything that overflowed (inf) or was computed from an undefined reference
-    // (NaN) fails the comparison.  Only then the wave takes the slow path, which brings the
-    // reference up to the true running maximum and rescales O and l.
-    uint32_t pk[2][8];
-    float ts[2];
-    exp_pack_sum(s, c, st.mc, pk, ts);
-    const bool ok = (ts[0] <= kTrip) & (ts[1] <= kTrip);
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!ok) != 0, 0)) {
-        float mcu[2];
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-            float mx = fmax2(s[nb][0], s[nb][1]);
-#pragma unroll
-            for (int r = 2; r < 16; r += 2) mx = fmax2(mx, fmax2(s[nb][r], s[nb][r + 1]));
-            mx = pair_max(mx);
-            const float m_old = st.m[nb];
-            const float m_new = fmax2(m_old, mx);
-            // m_new == -inf: every key so far carried a -inf additive mask.  Nothing has been
-            // accumulated yet, this sub-tile contributes zeros, and the stored reference stays
-            // undefined (+inf) so that the next sub-tile comes back here.
-            const bool empty = m_new == -__builtin_inff();
-            const float alpha = empty ? 1.f : __builtin_amdgcn_exp2f((m_old - m_new) * c);
-            st.l[nb] *= alpha;
-            scale_accumulators<G::DB>(st.o, nb, alpha);
-            st.m[nb] = m_new;
-            st.mc[nb] = empty ? __builtin_inff() : -m_new * c;
-            mcu[nb] = empty ? 0.f : -m_new * c;
-        }
-        exp_pack_sum(s, c, mcu, pk, ts);
-    }
-    st.l[0] += ts[0];
-    st.l[1] += ts[1];
-
-    // ---- O^T += V_sub^T * P^T ------------------------------------------------------------
-    // Transpose read: inside each group of 16 lanes, lane j receives, for i = 0..3, element
-    // (j % 4) of the 8-byte row fetched by lane 4 i + j / 4.  With lane s of a group pointing at
-    // V[key0 + s / 4][d0 + 4 (s % 4) ...], lane j ends up with V[key0 + i][d0 + j], i = 0..3.
-    const int s16 = lane & 15;
-    const _Float16* vrow = vs + (sub * 32 + 4 * g + (s16 >> 2)) * G::VSTR + 16 * ((lane >> 4) & 1) +
-                           4 * (s16 & 3);
+// O^T += V_sub^T * P^T.  k-slot (g, i) of k-step t is key 16 t + 8 (i / 4) + 4 g + i % 4 on both
+// operands: that is where the packed P^T registers (accumulator rows 8 t .. 8 t + 7) come from, and
+// the two transpose reads fetch keys 16 t + 4 g + {0..3} and 16 t + 8 + 4 g + {0..3}.
+template <int H>
+__device__ __forceinline__ void pv_mfma(floatx16 (&o)[Geometry<H>::DB][2], const _Float16* vrow,
+                                        const uint32_t (&pk)[2][8]) {
+    using G = Geometry<H>;
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         half8 pb[2];
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
-            u32x4 w = {pk[nb][4 * t], pk[nb][4 * t + 1], pk[nb][4 * t + 2], pk[nb][4 * t + 3]};
+            const u32x4 w = {pk[nb][4 * t], pk[nb][4 * t + 1], pk[nb][4 * t + 2], pk[nb][4 * t + 3]};
             pb[nb] = __builtin_bit_cast(half8, w);
         }
 #pragma unroll
@@ -328,20 +259,221 @@ __device__ __forceinline__ void process_subtile(WaveState<H>& st, const _Float16
             const half8 a = __builtin_bit_cast(half8, both);
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb)
-                st.o[db][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[nb], st.o[db][nb], 0, 0, 0);
+                o[db][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[nb], o[db][nb], 0, 0, 0);
         }
     }
 }
 
+// Slow path of the online softmax: bring the reference up to the true running maximum of the rows,
+// rescale O and l, and redo the exponentials of this sub-tile against the new reference.
+template <int H>
+__device__ __forceinline__ void softmax_fix(WaveState<H>& st, const floatx16 (&s)[2], float c,
+                                         uint32_t (&pk)[2][8], float (&ts)[2]) {
+    using G = Geometry<H>;
+    float mcu[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+        float mx = fmax2(s[nb][0], s[nb][1]);
+#pragma unroll
+        for (int r = 2; r < 16; r += 2) mx = fmax2(mx, fmax2(s[nb][r], s[nb][r + 1]));
+        mx = pair_max(mx);
+        const float m_old = st.m[nb];
+        const float m_new = fmax2(m_old, mx);
+        // m_new == -inf: every key so far carried a -inf additive mask.  Nothing has been
+        // accumulated yet, this sub-tile contributes zeros, and the stored reference stays
+        // undefined (+inf) so that the next sub-tile comes back here.
+        const bool empty = m_new == -__builtin_inff();
+        const float alpha = empty ? 1.f : __builtin_amdgcn_exp2f((m_old - m_new) * c);
+        st.l[nb] *= alpha;
+        scale_accumulators<G::DB>(st.o, nb, alpha);
+        st.m[nb] = m_new;
+        st.mc[nb] = empty ? __builtin_inff() : -m_new * c;
+        mcu[nb] = empty ? 0.f : -m_new * c;
+    }
+    exp_pack_sum(s, c, mcu, pk, ts);
+}
+
+// Fast path: exponentiate against the reference maximum of the rows seen so far, without looking
+// at this sub-tile's maximum.  Any reference works as long as numerator and denominator share it;
+// it only has to keep exp2 inside the fp16 range.  Each lane checks that with its own partial row
+// sum: 16 non-negative terms whose sum is <= kTrip are each <= kTrip, and anything that overflowed
+// (inf) or was computed from an undefined reference (NaN) fails the comparison.  Only then the wave
+// takes the slow path.
+template <int H>
+__device__ __forceinline__ void softmax_check(WaveState<H>& st, const floatx16 (&s)[2], float c,
+                                              uint32_t (&pk)[2][8], float (&ts)[2]) {
+    const bool ok = (ts[0] <= kTrip) & (ts[1] <= kTrip);
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!ok) != 0, 0)) softmax_fix<H>(st, s, c, pk, ts);
+    st.l[0] += ts[0];
+    st.l[1] += ts[1];
+}
+
+// Processes 32 keys (one sub-tile) for the wave's 64 queries, one stage after the other.  Used for
+// the ragged last tile and for the additive-mask variant.
+//   ks/vs : LDS tile base for the current buffer
+//   nvalid: number of valid keys in this sub-tile (only read when MASKED)
+template <int H, bool MASKED, bool HAS_MASK>
+__device__ __forceinline__ void process_subtile(WaveState<H>& st, const _Float16* ks,
+                                                const _Float16* vs, int sub, int nvalid,
+                                                float c, int lane,
+                                                const _Float16* mask_row0, const _Float16* mask_row1,
+                                                int key_base, int L) {
+    const int g = lane >> 5;
+    floatx16 s[2];
+    qk_mfma<H>(s, st.q, k_operand_ptr<H>(ks, sub, lane));
+
+    if constexpr (HAS_MASK) {
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            const _Float16* mrow = nb == 0 ? mask_row0 : mask_row1;
+            if (mrow != nullptr) {
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    const int key = key_base + 8 * r4 + 4 * g;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (key + j < L) {
+                            // The mask is added to the scaled score; S holds raw scores, so the
+                            // mask is brought to raw units: s*scale + mask = scale*(s + mask/scale).
+                            s[nb][4 * r4 + j] += (float)mrow[key + j] * (1.4426950408889634f / c);
+                        }
+                    }
+                }
+            }
+        }
+    }
+    if constexpr (MASKED) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+            if (key >= nvalid) {
+                s[0][r] = -__builtin_inff();
+                s[1][r] = -__builtin_inff();
+            }
+        }
+    }
+
+    uint32_t pk[2][8];
+    float ts[2];
+    exp_pack_sum(s, c, st.mc, pk, ts);
+    softmax_check<H>(st, s, c, pk, ts);
+    pv_mfma<H>(st.o, v_operand_ptr<H>(vs, sub, lane), pk);
+}
+
+// One stage of the software pipeline: three independent pieces of work on three sub-tiles,
+//   s_next = K_{j+1} Q^T          (matrix core)
+//   p_cur  = exp2(s_cur ...)      (vector ALU)
+//   O^T   += V_{j-1}^T p_prev     (matrix core)
+// written out in the order the instructions should issue: the exponentials are cut into 16 chunks
+// of one fp16 pair (2 fma, 2 exp, 1 pack, 1 dot2: about the duration of one 32x32x16 MFMA), each
+// followed by its share of the matrix instructions, with the LDS operand reads issued PF operands
+// ahead of their use.  A scheduling barrier after every chunk keeps the compiler from regrouping
+// them, so that one wave by itself keeps the matrix core and the vector ALU busy together.
+template <int H>
+__device__ __forceinline__ void pipeline_stage(WaveState<H>& st, floatx16 (&s_next)[2],
+                                               const floatx16 (&s_cur)[2], uint32_t (&p_cur)[2][8],
+                                               const uint32_t (&p_prev)[2][8], const _Float16* krow,
+                                               const _Float16* vrow, float c) {
+    using G = Geometry<H>;
+    constexpr int NQK = G::KS;            // operand slots of the first product (K rows)
+    constexpr int NPV = 2 * G::DB;        // operand slots of the second product (V^T blocks)
+    constexpr int NU = NQK + NPV;
+    constexpr int NM = 2 * NU;            // matrix instructions of this stage
+    constexpr int D = 2;                  // chunks of vector work issued before the first MFMA
+    constexpr int PF = NU < 3 ? NU : 3;   // operand slots fetched ahead
+    typedef short short8v __attribute__((ext_vector_type(8)));
+
+    half8 opnd[NU];
+    auto fetch = [&](int u) {
+        if (u < NQK) {
+            opnd[u] = *reinterpret_cast<const half8*>(krow + u * 16);
+        } else {
+            const int t = (u - NQK) / G::DB, db = (u - NQK) % G::DB;
+            const _Float16* p0 = vrow + (16 * t) * G::VSTR + db * 32;
+            const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS short4v*)(p0));
+            const short4v hi =
+                __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS short4v*)(p0 + 8 * G::VSTR));
+            const short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            opnd[u] = __builtin_bit_cast(half8, both);
+        }
+    };
+    auto mma = [&](int j) {
+        const int u = j >> 1, nb = j & 1;
+        if (u < NQK) {
+            if (u == 0) {
+                floatx16 z;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) z[r] = 0.f;
+                s_next[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(opnd[u], st.q[nb][u], z, 0, 0, 0);
+            } else {
+                s_next[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(opnd[u], st.q[nb][u], s_next[nb], 0, 0, 0);
+            }
+        } else {
+            const int t = (u - NQK) / G::DB, db = (u - NQK) % G::DB;
+            const u32x4 w = {p_prev[nb][4 * t], p_prev[nb][4 * t + 1], p_prev[nb][4 * t + 2],
+                             p_prev[nb][4 * t + 3]};
+            st.o[db][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(opnd[u], __builtin_bit_cast(half8, w),
+                                                                  st.o[db][nb], 0, 0, 0);
+        }
+    };
+
+    const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+    float ts[2] = {0.f, 0.f};
+    float e0 = 0.f, e1 = 0.f;   // exponentials of the previous chunk, packed one chunk later
+
+#pragma unroll
+    for (int u = 0; u < PF; ++u) fetch(u);
+#pragma unroll
+    for (int i = 0; i <= 16; ++i) {
+        if (i < 16) {
+            const int nb = i >> 3, r = (i & 7) * 2;
+            const float a0 = __builtin_fmaf(s_cur[nb][r], c, st.mc[nb]);
+            const float a1 = __builtin_fmaf(s_cur[nb][r + 1], c, st.mc[nb]);
+            const float n0 = __builtin_amdgcn_exp2f(a0);
+            const float n1 = __builtin_amdgcn_exp2f(a1);
+            if (i > 0) {
+                const int pnb = (i - 1) >> 3, pr2 = (i - 1) & 7;
+                const uint32_t pp = pack_rtz(e0, e1);
+                p_cur[pnb][pr2] = pp;
+                ts[pnb] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, pp), ones, ts[pnb], false);
+            }
+            e0 = n0;
+            e1 = n1;
+        } else {
+            const uint32_t pp = pack_rtz(e0, e1);
+            p_cur[1][7] = pp;
+            ts[1] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, pp), ones, ts[1], false);
+        }
+        if (i >= D) {
+            const int jlo = (i - D) * NM / 16;
+            const int jhi = i == 16 ? NM : (i - D + 1) * NM / 16;
+#pragma unroll
+            for (int j = jlo; j < jhi; ++j) {
+                mma(j);
+                if ((j & 1) == 0 && (j >> 1) + PF < NU) fetch((j >> 1) + PF);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    softmax_check<H>(st, s_cur, c, p_cur, ts);
+}
+
+#ifndef FA_WAVES_PER_EU_64
+#define FA_WAVES_PER_EU_64 2
+#endif
+
 template <int H, int NW, int BK, bool HAS_MASK>
-__global__ __launch_bounds__(NW * 64, (H <= 64 ? 2 : 1)) void fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(NW * 64, (H <= 64 ? FA_WAVES_PER_EU_64 : 1)) void fwd_kernel(const FwdParams p) {
     using G = Geometry<H>;
     constexpr int BQ = NW * 64;
     constexpr int NSUB = BK / 32;
+    static_assert(BK == 64, "the pipelined loop is written for two sub-tiles per tile");
 
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[];
     _Float16* const ks_base = smem;                                // [2][BK][KSTR]
     _Float16* const vs_base = smem + 2 * BK * G::KSTR;             // [2][BK][VSTR]
+    constexpr int KTILE = BK * G::KSTR;
+    constexpr int VTILE = BK * G::VSTR;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -369,7 +501,7 @@ __global__ __launch_bounds__(NW * 64, (H <= 64 ? 2 : 1)) void fwd_kernel(const F
 
     // V columns beyond H (only when H = 16) stay zero for the whole kernel.
     if constexpr (G::HV != H) {
-        for (int i = tid; i < 2 * BK * G::VSTR; i += BQ) vs_base[i] = (_Float16)0.f;
+        for (int i = tid; i < 2 * VTILE; i += BQ) vs_base[i] = (_Float16)0.f;
         __syncthreads();
     }
 
@@ -393,49 +525,109 @@ __global__ __launch_bounds__(NW * 64, (H <= 64 ? 2 : 1)) void fwd_kernel(const F
             for (int r = 0; r < 16; ++r) st.o[db][nb][r] = 0.f;
     }
 
-    const _Float16* mask_row0 = nullptr;
-    const _Float16* mask_row1 = nullptr;
+    const int ntiles = (L + BK - 1) / BK;
+    const int nfull = L / BK;
+    const float c = p.scale_log2e;
+    const int64_t sl = p.stride_l;
+    TileLoader<H, NW, BK> loader;
+
     if constexpr (HAS_MASK) {
+        // Additive-mask variant: plain double-buffered loop, one sub-tile after the other.
+        const _Float16* mask_row0 = nullptr;
+        const _Float16* mask_row1 = nullptr;
         const _Float16* mb = p.mask + (int64_t)b * L * L;
         if (q0 + ln < L) mask_row0 = mb + (int64_t)(q0 + ln) * L;
         if (q0 + 32 + ln < L) mask_row1 = mb + (int64_t)(q0 + 32 + ln) * L;
-    }
 
-    const int ntiles = (L + BK - 1) / BK;
-    const float c = p.scale_log2e;
-
-    TileLoader<H, NW, BK> loader;
-    loader.load(kbase, vbase, p.stride_l, 0, L, tid);
-    loader.store(ks_base, vs_base, tid);
-    __syncthreads();
-
-    // Full tiles: one straight path per iteration.  The ragged last tile, if any, is peeled off so
-    // that its masking code does not share a loop (and register assignment) with the hot path.
-    const int nfull = L / BK;
-    for (int t = 0; t < nfull; ++t) {
-        const int buf = t & 1;
-        const _Float16* ks = ks_base + buf * BK * G::KSTR;
-        const _Float16* vs = vs_base + buf * BK * G::VSTR;
-        const bool has_next = t + 1 < ntiles;
-        if (has_next) loader.load(kbase, vbase, p.stride_l, (t + 1) * BK, L, tid);
-#pragma unroll
-        for (int sub = 0; sub < NSUB; ++sub)
-            process_subtile<H, false, HAS_MASK>(st, ks, vs, sub, 32, c, lane, mask_row0, mask_row1,
-                                                t * BK + sub * 32, L);
-        if (has_next) loader.store(ks_base + (buf ^ 1) * BK * G::KSTR, vs_base + (buf ^ 1) * BK * G::VSTR, tid);
+        loader.load_k(kbase, sl, 0, L, tid);
+        loader.load_v(vbase, sl, 0, L, tid);
+        loader.store_k(ks_base, tid);
+        loader.store_v(vs_base, tid);
         __syncthreads();
-    }
-    if (nfull < ntiles) {
-        const int buf = nfull & 1;
-        const _Float16* ks = ks_base + buf * BK * G::KSTR;
-        const _Float16* vs = vs_base + buf * BK * G::VSTR;
-        const int key0 = nfull * BK;
+        for (int t = 0; t < ntiles; ++t) {
+            const int buf = t & 1;
+            const bool has_next = t + 1 < ntiles;
+            if (has_next) {
+                loader.load_k(kbase, sl, (t + 1) * BK, L, tid);
+                loader.load_v(vbase, sl, (t + 1) * BK, L, tid);
+            }
 #pragma unroll
-        for (int sub = 0; sub < NSUB; ++sub) {
-            const int nvalid = L - key0 - sub * 32;
-            if (nvalid > 0)
-                process_subtile<H, true, HAS_MASK>(st, ks, vs, sub, nvalid, c, lane, mask_row0, mask_row1,
-                                                   key0 + sub * 32, L);
+            for (int sub = 0; sub < NSUB; ++sub) {
+                const int nvalid = L - t * BK - sub * 32;
+                if (nvalid > 0)
+                    process_subtile<H, true, true>(st, ks_base + buf * KTILE, vs_base + buf * VTILE, sub,
+                                                   nvalid, c, lane, mask_row0, mask_row1,
+                                                   t * BK + sub * 32, L);
+            }
+            if (has_next) {
+                loader.store_k(ks_base + (buf ^ 1) * KTILE, tid);
+                loader.store_v(vs_base + (buf ^ 1) * VTILE, tid);
+            }
+            __syncthreads();
+        }
+    } else {
+        // Software pipeline over the full tiles.  With j the sub-tile index, stage j issues
+        // QK^T of sub-tile j + 1, the exponentials of sub-tile j and PV of sub-tile j - 1, so K runs
+        // one tile ahead of V: iteration T of the loop below reads K tile T + 1 and V tile T and
+        // refills the other K buffer with tile T + 2 and the other V buffer with tile T + 1.
+        loader.load_k(kbase, sl, 0, L, tid);
+        loader.load_v(vbase, sl, 0, L, tid);
+        loader.store_k(ks_base, tid);
+        loader.store_v(vs_base, tid);
+        loader.load_k(kbase, sl, BK, L, tid);
+        loader.store_k(ks_base + KTILE, tid);
+        __syncthreads();
+
+        const bool ragged = nfull < ntiles;
+        if (nfull > 0) {
+            floatx16 sa[2], sb[2];
+            uint32_t pa[2][8], pb[2][8];
+            float ts[2];
+            // stage 0 (no PV yet)
+            qk_mfma<H>(sa, st.q, k_operand_ptr<H>(ks_base, 0, lane));
+            qk_mfma<H>(sb, st.q, k_operand_ptr<H>(ks_base, 1, lane));
+            exp_pack_sum(sa, c, st.mc, pa, ts);
+            softmax_check<H>(st, sa, c, pa, ts);
+            // every wave is done with K tile 0 before anyone overwrites its buffer
+            __syncthreads();
+
+            for (int T = 0; T + 1 < nfull; ++T) {
+                const _Float16* kcur = ks_base + ((T + 1) & 1) * KTILE;
+                const _Float16* vcur = vs_base + (T & 1) * VTILE;
+                loader.load_k(kbase, sl, (T + 2) * BK, L, tid);
+                loader.load_v(vbase, sl, (T + 1) * BK, L, tid);
+                pipeline_stage<H>(st, sa, sb, pb, pa, k_operand_ptr<H>(kcur, 0, lane),
+                                  v_operand_ptr<H>(vcur, 0, lane), c);
+                pipeline_stage<H>(st, sb, sa, pa, pb, k_operand_ptr<H>(kcur, 1, lane),
+                                  v_operand_ptr<H>(vcur, 1, lane), c);
+                loader.store_k(ks_base + (T & 1) * KTILE, tid);
+                loader.store_v(vs_base + ((T + 1) & 1) * VTILE, tid);
+                __syncthreads();
+            }
+
+            // drain: exponentials of the last full sub-tile, PV of the last two
+            const _Float16* vlast = vs_base + ((nfull - 1) & 1) * VTILE;
+            if (ragged) loader.load_v(vbase, sl, nfull * BK, L, tid);
+            // (PV of sub-tile j - 1 goes first: a rescale triggered by sub-tile j must see it in O)
+            pv_mfma<H>(st.o, v_operand_ptr<H>(vlast, 0, lane), pa);
+            exp_pack_sum(sb, c, st.mc, pb, ts);
+            softmax_check<H>(st, sb, c, pb, ts);
+            pv_mfma<H>(st.o, v_operand_ptr<H>(vlast, 1, lane), pb);
+            if (ragged) {
+                loader.store_v(vs_base + (nfull & 1) * VTILE, tid);
+                __syncthreads();
+            }
+        }
+        if (ragged) {
+            const int buf = nfull & 1;
+            const int key0 = nfull * BK;
+#pragma unroll
+            for (int sub = 0; sub < NSUB; ++sub) {
+                const int nvalid = L - key0 - sub * 32;
+                if (nvalid > 0)
+                    process_subtile<H, true, false>(st, ks_base + buf * KTILE, vs_base + buf * VTILE, sub,
+                                                    nvalid, c, lane, nullptr, nullptr, key0 + sub * 32, L);
+            }
         }
     }
 
