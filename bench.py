@@ -22,6 +22,12 @@ if REPO not in sys.path:
 
 PEAK_TFLOPS_FP16 = 2500.0   # MI355X dense fp16 MFMA, published
 
+# HBM bytes per launch of the forward kernel, measured with rocprofv3 (FETCH_SIZE and WRITE_SIZE
+# in separate --pmc runs of this script, each scaled by what the same counter reads for the 1 GiB
+# calibration copy below: 2.000 for fetch, 1.000 for write).  Summaries: profiles/fwd_kernel_c3.md
+# and profiles/fwd_kernel_c4.md.
+MEASURED_TRAFFIC_BYTES = {"c3": 134.4e6, "c4": 813.3e6}
+
 
 def cpu_baseline(w, q, k, v, gpu_out, budget_s):
     """Naive float32 attention on the host cores for a bounded sample of (batch, head) pairs.
@@ -65,6 +71,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c3")
+    ap.add_argument("--calibration-copy-mib", type=int, default=1024,
+                    help="size of the plain copy run before the timed region (0 disables it)")
     ap.add_argument("--cpu-budget-s", type=float, default=15.0,
                     help="seconds of host time for the CPU baseline sample (0 disables it)")
     args = ap.parse_args()
@@ -85,6 +93,16 @@ def main():
     q, k, v = workloads.make_inputs(w)
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     chunk = min(128, w.H * 2)
+
+    # A plain device-to-device copy of known size, outside the timed region: the reference point
+    # against which the HBM counters (FETCH_SIZE / WRITE_SIZE) of a profiler run are scaled.
+    if args.calibration_copy_mib > 0:
+        src = torch.arange(args.calibration_copy_mib * (1 << 18), dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         out = fused_attn.attention_forward(w.H, chunk, qd, kd, vd)
@@ -128,7 +146,7 @@ def main():
             "peak": PEAK_TFLOPS_FP16,
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_TFLOPS_FP16,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
             "kernel_ms": kernel_ms,
         },
     }

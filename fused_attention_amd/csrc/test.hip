@@ -5,7 +5,9 @@
 // but checks sampled output rows against a double-precision host evaluation of
 // softmax(Q K^T / sqrt(H)) V and exits non-zero when the error exceeds the tolerance.
 //
-// usage: fa_test [B R L H [iters [blhd|bhld [input_scale]]]]
+// usage: fa_test [B R L H [iters [blhd|bhld [input_scale [qzero|vconst|vcol]]]]]
+//        fa_test mfma-peak        what v_mfma_f32_32x32x16_f16 sustains on this chip with zero
+//                                 operands and with N(0,1) operands (the rate depends on the data)
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -29,6 +31,79 @@
 
 namespace {
 
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// Back-to-back matrix instructions on four independent accumulators, two waves per SIMD on every
+// compute unit: the ceiling any fp16 MFMA kernel on this chip is measured against.
+__global__ __launch_bounds__(512) void mfma_peak_kernel(float* out, const half8* data, int iters) {
+    half8 a[4], b[4];
+    for (int i = 0; i < 4; i++) {
+        a[i] = data[threadIdx.x + i * 512];
+        b[i] = data[threadIdx.x + (i + 4) * 512];
+    }
+    floatx16 c[4];
+    for (int n = 0; n < 4; n++)
+        for (int r = 0; r < 16; r++) c[n][r] = 0.f;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int j = 0; j < 16; j++)
+            c[j % 4] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j % 4], b[(j / 4) % 4], c[j % 4], 0, 0, 0);
+    }
+    float s = 0.f;
+    for (int n = 0; n < 4; n++)
+        for (int r = 0; r < 16; r++) s += c[n][r];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+int mfma_peak() {
+    hipDeviceProp_t prop;
+    HIP_OK(hipGetDeviceProperties(&prop, 0));
+    const int blocks = prop.multiProcessorCount, threads = 512, iters = 20000;
+    const size_t n = 512 * 8 * 8;
+    std::vector<_Float16> zeros(n, (_Float16)0.f), normal(n);
+    uint32_t s = 12345u;
+    for (auto& x : normal) {  // sum of 12 uniforms - 6: close to N(0,1)
+        float u = 0.f;
+        for (int q = 0; q < 12; ++q) {
+            s = s * 1664525u + 1013904223u;
+            u += (float)(s >> 8) / 16777216.0f;
+        }
+        x = (_Float16)(u - 6.0f);
+    }
+    half8 *dz, *dn;
+    float* out;
+    HIP_OK(hipMalloc(&dz, n * 2));
+    HIP_OK(hipMalloc(&dn, n * 2));
+    HIP_OK(hipMalloc(&out, (size_t)blocks * threads * 4));
+    HIP_OK(hipMemcpy(dz, zeros.data(), n * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dn, normal.data(), n * 2, hipMemcpyHostToDevice));
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    for (int rep = 0; rep < 2; ++rep) {
+        for (int kind = 0; kind < 2; ++kind) {
+            const half8* d = kind == 0 ? dz : dn;
+            hipLaunchKernelGGL(mfma_peak_kernel, dim3(blocks), dim3(threads), 0, nullptr, out, d, 200);
+            HIP_OK(hipEventRecord(e0, nullptr));
+            for (int r = 0; r < 3; ++r)
+                hipLaunchKernelGGL(mfma_peak_kernel, dim3(blocks), dim3(threads), 0, nullptr, out, d, iters);
+            HIP_OK(hipEventRecord(e1, nullptr));
+            HIP_OK(hipEventSynchronize(e1));
+            float ms = 0.f;
+            HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+            ms /= 3.f;
+            const double flop = (double)blocks * (threads / 64) * iters * 16.0 * 32768.0;
+            std::printf("mfma-peak %-16s %d CUs x 8 waves: %.3f ms per launch, %.0f TFLOP/s\n",
+                        kind == 0 ? "zero operands" : "N(0,1) operands", blocks, ms, flop / ms / 1e9);
+        }
+    }
+    (void)hipFree(dz);
+    (void)hipFree(dn);
+    (void)hipFree(out);
+    return 0;
+}
+
 // Values in [-amp, amp) from a 16-bit multiplicative generator, rounded to fp16.
 void fill_values(std::vector<_Float16>& dst, uint32_t seed, float amp) {
     uint32_t s = seed;
@@ -45,6 +120,7 @@ int main(int argc, char** argv) {
     int iters = 20;
     bool bhld = false;
     float amp = 1.7320508f;  // uniform with unit variance
+    if (argc >= 2 && std::strcmp(argv[1], "mfma-peak") == 0) return mfma_peak();
     if (argc >= 5) {
         B = std::atoll(argv[1]);
         R = std::atoll(argv[2]);
