@@ -68,8 +68,8 @@ def cpu_baseline(w, q, k, v, gpu_out, budget_s):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="c3")
     ap.add_argument("--calibration-copy-mib", type=int, default=1024,
                     help="size of the plain copy run before the timed region (0 disables it)")

@@ -13,20 +13,35 @@ namespace {
 constexpr int kKeyTile = 64;     // keys per LDS tile
 constexpr int kNumCu = 256;      // compute units of one MI355X
 
-// Wave64s per workgroup (64 query rows each).  Eight waves share one K/V stream between twice
-// as many queries, which pays once there are enough workgroups to give every compute unit two of
-// them; head_dim 128 needs the whole register file of a SIMD for one wave, so it stays at four.
-int pick_waves(int64_t B, int64_t R, int64_t L, int64_t H) {
-    if (H > 64) return 4;
-    const int64_t wgs8 = B * R * ((L + 511) / 512);
-    return wgs8 >= 2 * kNumCu ? 8 : 4;
+// Launch shape: wave64s per workgroup, blocks of 32 query rows per wave, waves per SIMD the
+// registers are budgeted for.
+struct Shape {
+    int waves;
+    int nqb;
+    int rows() const { return waves * 32 * nqb; }
+};
+
+// Three shapes, picked by how many workgroups the problem gives the 256 compute units:
+//   {8, 2}  eight 64-row waves share one K/V stream between 512 queries: best once every compute
+//           unit still gets two such workgroups (head_dim <= 64, two waves per SIMD);
+//   {4, 2}  four 64-row waves, 256 queries per workgroup;
+//   {4, 1}  four 32-row waves, 128 queries per workgroup, three (head_dim <= 64) or two
+//           (head_dim 128) waves per SIMD: more, smaller workgroups for short sequences.
+// head_dim 128 with 64-row waves needs the whole register file of a SIMD for one wave.
+Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask) {
+    // the additive-mask variant at head_dim 128 only exists with 32-row waves (register budget)
+    if (H > 64 && has_mask) return {4, 1};
+    const int64_t wgs512 = B * R * ((L + 511) / 512);
+    const int64_t wgs256 = B * R * ((L + 255) / 256);
+    if (H > 64) return wgs256 >= 6 * kNumCu ? Shape{4, 2} : Shape{4, 1};
+    if (wgs512 >= 2 * kNumCu) return {8, 2};
+    return wgs256 >= 2 * kNumCu ? Shape{4, 2} : Shape{4, 1};
 }
 
-template <int H, int NW, bool HAS_MASK>
+template <int H, int NW, int NQB, int WPE, bool HAS_MASK>
 hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
-    constexpr int kWaves = NW;
-    constexpr int lds = fa::lds_bytes<H, kWaves, kKeyTile>();
-    auto kernel = fa::fwd_kernel<H, kWaves, kKeyTile, HAS_MASK>;
+    constexpr int lds = fa::lds_bytes<H, NW, kKeyTile>();
+    auto kernel = fa::fwd_kernel<H, NW, kKeyTile, NQB, WPE, HAS_MASK>;
     // Dynamic LDS above 64 KiB has to be opted into once per kernel function.
     if constexpr (lds > 64 * 1024) {
         static std::once_flag once;
@@ -38,17 +53,30 @@ hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
         if (attr_status != hipSuccess) return attr_status;
     }
     const int grid = p.wgs_per_xcd * fa::kNumXcd;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kWaves * 64), lds, stream, p);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * 64), lds, stream, p);
     return hipGetLastError();
 }
 
+template <int H, bool HAS_MASK>
+hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) {
+    if constexpr (H > 64) {
+        if constexpr (HAS_MASK)
+            return launch<H, 4, 1, 2, true>(p, stream);
+        else
+            return sh.nqb == 2 ? launch<H, 4, 2, 1, false>(p, stream) : launch<H, 4, 1, 2, false>(p, stream);
+    } else {
+        if (sh.waves == 8) return launch<H, 8, 2, 2, HAS_MASK>(p, stream);
+        return sh.nqb == 2 ? launch<H, 4, 2, 2, HAS_MASK>(p, stream) : launch<H, 4, 1, 3, HAS_MASK>(p, stream);
+    }
+}
+
 template <bool HAS_MASK>
-hipError_t dispatch(int64_t H, int waves, const fa::FwdParams& p, hipStream_t stream) {
+hipError_t dispatch(int64_t H, Shape sh, const fa::FwdParams& p, hipStream_t stream) {
     switch (H) {
-        case 16: return waves == 8 ? launch<16, 8, HAS_MASK>(p, stream) : launch<16, 4, HAS_MASK>(p, stream);
-        case 32: return waves == 8 ? launch<32, 8, HAS_MASK>(p, stream) : launch<32, 4, HAS_MASK>(p, stream);
-        case 64: return waves == 8 ? launch<64, 8, HAS_MASK>(p, stream) : launch<64, 4, HAS_MASK>(p, stream);
-        case 128: return launch<128, 4, HAS_MASK>(p, stream);
+        case 16: return dispatch_shape<16, HAS_MASK>(sh, p, stream);
+        case 32: return dispatch_shape<32, HAS_MASK>(sh, p, stream);
+        case 64: return dispatch_shape<64, HAS_MASK>(sh, p, stream);
+        case 128: return dispatch_shape<128, HAS_MASK>(sh, p, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -57,7 +85,7 @@ bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u
 
 int validate(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,
              int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h, int64_t stride_l,
-             fa::FwdParams* p, float scale, int* waves) {
+             fa::FwdParams* p, float scale, Shape* shape) {
     if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return FA_ERR_NULL_POINTER;
     if (!fa_fwd_query(H)) return FA_ERR_BAD_HEAD_DIM;
     if (B < 1 || R < 1 || L < 1) return FA_ERR_BAD_SHAPE;
@@ -67,8 +95,8 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     if (mask != nullptr && (reinterpret_cast<uintptr_t>(mask) & 1u) != 0) return FA_ERR_MISALIGNED;
     constexpr int64_t kMaxInt = 0x7fffffff;
     if (L > kMaxInt - 4096 || B > kMaxInt || R > kMaxInt) return FA_ERR_TOO_LARGE;
-    *waves = pick_waves(B, R, L, H);
-    const int64_t bq = *waves * 64;
+    *shape = pick_shape(B, R, L, H, mask != nullptr);
+    const int64_t bq = shape->rows();
     const int64_t n_qtiles = (L + bq - 1) / bq;
     const int64_t total = B * R * n_qtiles;
     if (total > kMaxInt - 8 || B * R > kMaxInt) return FA_ERR_TOO_LARGE;
@@ -121,11 +149,11 @@ int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* 
            int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h, int64_t stride_l,
            float scale, void* stream) {
     fa::FwdParams p;
-    int waves = 4;
-    const int rc = validate(q, k, v, mask, out, B, R, L, H, stride_b, stride_h, stride_l, &p, scale, &waves);
+    Shape shape{4, 2};
+    const int rc = validate(q, k, v, mask, out, B, R, L, H, stride_b, stride_h, stride_l, &p, scale, &shape);
     if (rc != FA_OK) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const hipError_t e = mask != nullptr ? dispatch<true>(H, waves, p, s) : dispatch<false>(H, waves, p, s);
+    const hipError_t e = mask != nullptr ? dispatch<true>(H, shape, p, s) : dispatch<false>(H, shape, p, s);
     return static_cast<int>(e);
 }
 

@@ -149,14 +149,15 @@ struct TileLoader {
 // Largest partial row sum (16 terms) the fast path of the online softmax accepts.
 constexpr float kTrip = 16384.f;
 
-// p = exp2(s * c + mc) for the 2 x 16 scores of a sub-tile, rounded to fp16 pairs (round toward
+// p = exp2(s * c + mc) for the NQB x 16 scores of a sub-tile, rounded to fp16 pairs (round toward
 // zero), and the per-lane sums of the rounded values.  The sums are taken over the rounded
 // probabilities that enter the second product, so numerator and denominator see the same rounding.
-__device__ __forceinline__ void exp_pack_sum(const floatx16 (&s)[2], float c, const float (&mc)[2],
-                                             uint32_t (&pk)[2][8], float (&ts)[2]) {
+template <int NQB>
+__device__ __forceinline__ void exp_pack_sum(const floatx16 (&s)[NQB], float c, const float (&mc)[NQB],
+                                             uint32_t (&pk)[NQB][8], float (&ts)[NQB]) {
     const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int nb = 0; nb < NQB; ++nb) {
         float acc = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
@@ -174,8 +175,8 @@ __device__ __forceinline__ void exp_pack_sum(const floatx16 (&s)[2], float c, co
 // as input and output, so that the rarely taken rescale does not make the compiler keep a second
 // copy of the accumulators (and copy them on the common path).  The leading wait covers the
 // matrix-core results the multiplies read.
-template <int DB>
-__device__ __forceinline__ void scale_accumulators(floatx16 (&o)[DB][2], int nb, float alpha) {
+template <int DB, int NQB>
+__device__ __forceinline__ void scale_accumulators(floatx16 (&o)[DB][NQB], int nb, float alpha) {
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
@@ -188,15 +189,16 @@ __device__ __forceinline__ void scale_accumulators(floatx16 (&o)[DB][2], int nb,
     }
 }
 
-// Per-wave state: Q^T as B operands, O^T accumulators, online-softmax (m, l).
-template <int H>
+// Per-wave state for NQB blocks of 32 queries: Q^T as B operands, O^T accumulators,
+// online-softmax (m, l).
+template <int H, int NQB>
 struct WaveState {
     using G = Geometry<H>;
-    half8 q[2][G::KS];
-    floatx16 o[G::DB][2];
-    float m[2];   // reference row maximum of the raw (unscaled) scores, identical in lanes l and l^32
-    float mc[2];  // -m * c, the additive term of the exponent; +inf while no reference exists yet
-    float l[2];   // running sum of exp over the keys this lane has seen (half of each tile)
+    half8 q[NQB][G::KS];
+    floatx16 o[G::DB][NQB];
+    float m[NQB];   // reference row maximum of the raw (unscaled) scores, identical in lanes l and l^32
+    float mc[NQB];  // -m * c, the additive term of the exponent; +inf while no reference exists yet
+    float l[NQB];   // running sum of exp over the keys this lane has seen (half of each tile)
 };
 
 // LDS address of this lane's K row for sub-tile `sub` of a tile: A operand of S^T = K_sub * Q^T.
@@ -216,19 +218,19 @@ __device__ __forceinline__ const _Float16* v_operand_ptr(const _Float16* vs, int
            4 * (s16 & 3);
 }
 
-// S^T = K_sub * Q^T for 32 keys and the wave's 2 x 32 queries.
-template <int H>
-__device__ __forceinline__ void qk_mfma(floatx16 (&s)[2], const half8 (&q)[2][Geometry<H>::KS],
+// S^T = K_sub * Q^T for 32 keys and the wave's NQB x 32 queries.
+template <int H, int NQB>
+__device__ __forceinline__ void qk_mfma(floatx16 (&s)[NQB], const half8 (&q)[NQB][Geometry<H>::KS],
                                         const _Float16* krow) {
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+    for (int nb = 0; nb < NQB; ++nb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[nb][r] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < Geometry<H>::KS; ++kk) {
         const half8 a = *reinterpret_cast<const half8*>(krow + kk * 16);
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb)
+        for (int nb = 0; nb < NQB; ++nb)
             s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, q[nb][kk], s[nb], 0, 0, 0);
     }
 }
@@ -236,15 +238,15 @@ __device__ __forceinline__ void qk_mfma(floatx16 (&s)[2], const half8 (&q)[2][Ge
 // O^T += V_sub^T * P^T.  k-slot (g, i) of k-step t is key 16 t + 8 (i / 4) + 4 g + i % 4 on both
 // operands: that is where the packed P^T registers (accumulator rows 8 t .. 8 t + 7) come from, and
 // the two transpose reads fetch keys 16 t + 4 g + {0..3} and 16 t + 8 + 4 g + {0..3}.
-template <int H>
-__device__ __forceinline__ void pv_mfma(floatx16 (&o)[Geometry<H>::DB][2], const _Float16* vrow,
-                                        const uint32_t (&pk)[2][8]) {
+template <int H, int NQB>
+__device__ __forceinline__ void pv_mfma(floatx16 (&o)[Geometry<H>::DB][NQB], const _Float16* vrow,
+                                        const uint32_t (&pk)[NQB][8]) {
     using G = Geometry<H>;
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-        half8 pb[2];
+        half8 pb[NQB];
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
+        for (int nb = 0; nb < NQB; ++nb) {
             const u32x4 w = {pk[nb][4 * t], pk[nb][4 * t + 1], pk[nb][4 * t + 2], pk[nb][4 * t + 3]};
             pb[nb] = __builtin_bit_cast(half8, w);
         }
@@ -258,7 +260,7 @@ __device__ __forceinline__ void pv_mfma(floatx16 (&o)[Geometry<H>::DB][2], const
             const short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             const half8 a = __builtin_bit_cast(half8, both);
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb)
+            for (int nb = 0; nb < NQB; ++nb)
                 o[db][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[nb], o[db][nb], 0, 0, 0);
         }
     }
@@ -266,13 +268,13 @@ __device__ __forceinline__ void pv_mfma(floatx16 (&o)[Geometry<H>::DB][2], const
 
 // Slow path of the online softmax: bring the reference up to the true running maximum of the rows,
 // rescale O and l, and redo the exponentials of this sub-tile against the new reference.
-template <int H>
-__device__ __forceinline__ void softmax_fix(WaveState<H>& st, const floatx16 (&s)[2], float c,
-                                         uint32_t (&pk)[2][8], float (&ts)[2]) {
+template <int H, int NQB>
+__device__ __forceinline__ void softmax_fix(WaveState<H, NQB>& st, const floatx16 (&s)[NQB], float c,
+                                         uint32_t (&pk)[NQB][8], float (&ts)[NQB]) {
     using G = Geometry<H>;
-    float mcu[2];
+    float mcu[NQB];
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int nb = 0; nb < NQB; ++nb) {
         float mx = fmax2(s[nb][0], s[nb][1]);
 #pragma unroll
         for (int r = 2; r < 16; r += 2) mx = fmax2(mx, fmax2(s[nb][r], s[nb][r + 1]));
@@ -285,12 +287,12 @@ __device__ __forceinline__ void softmax_fix(WaveState<H>& st, const floatx16 (&s
         const bool empty = m_new == -__builtin_inff();
         const float alpha = empty ? 1.f : __builtin_amdgcn_exp2f((m_old - m_new) * c);
         st.l[nb] *= alpha;
-        scale_accumulators<G::DB>(st.o, nb, alpha);
+        scale_accumulators<G::DB, NQB>(st.o, nb, alpha);
         st.m[nb] = m_new;
         st.mc[nb] = empty ? __builtin_inff() : -m_new * c;
         mcu[nb] = empty ? 0.f : -m_new * c;
     }
-    exp_pack_sum(s, c, mcu, pk, ts);
+    exp_pack_sum<NQB>(s, c, mcu, pk, ts);
 }
 
 // Fast path: exponentiate against the reference maximum of the rows seen so far, without looking
@@ -299,33 +301,35 @@ __device__ __forceinline__ void softmax_fix(WaveState<H>& st, const floatx16 (&s
 // sum: 16 non-negative terms whose sum is <= kTrip are each <= kTrip, and anything that overflowed
 // (inf) or was computed from an undefined reference (NaN) fails the comparison.  Only then the wave
 // takes the slow path.
-template <int H>
-__device__ __forceinline__ void softmax_check(WaveState<H>& st, const floatx16 (&s)[2], float c,
-                                              uint32_t (&pk)[2][8], float (&ts)[2]) {
-    const bool ok = (ts[0] <= kTrip) & (ts[1] <= kTrip);
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!ok) != 0, 0)) softmax_fix<H>(st, s, c, pk, ts);
-    st.l[0] += ts[0];
-    st.l[1] += ts[1];
+template <int H, int NQB>
+__device__ __forceinline__ void softmax_check(WaveState<H, NQB>& st, const floatx16 (&s)[NQB], float c,
+                                              uint32_t (&pk)[NQB][8], float (&ts)[NQB]) {
+    bool ok = ts[0] <= kTrip;
+#pragma unroll
+    for (int nb = 1; nb < NQB; ++nb) ok = ok & (ts[nb] <= kTrip);
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!ok) != 0, 0)) softmax_fix<H, NQB>(st, s, c, pk, ts);
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) st.l[nb] += ts[nb];
 }
 
 // Processes 32 keys (one sub-tile) for the wave's 64 queries, one stage after the other.  Used for
 // the ragged last tile and for the additive-mask variant.
 //   ks/vs : LDS tile base for the current buffer
 //   nvalid: number of valid keys in this sub-tile (only read when MASKED)
-template <int H, bool MASKED, bool HAS_MASK>
-__device__ __forceinline__ void process_subtile(WaveState<H>& st, const _Float16* ks,
+template <int H, int NQB, bool MASKED, bool HAS_MASK>
+__device__ __forceinline__ void process_subtile(WaveState<H, NQB>& st, const _Float16* ks,
                                                 const _Float16* vs, int sub, int nvalid,
                                                 float c, int lane,
-                                                const _Float16* mask_row0, const _Float16* mask_row1,
+                                                const _Float16* const (&mask_row)[NQB],
                                                 int key_base, int L) {
     const int g = lane >> 5;
-    floatx16 s[2];
-    qk_mfma<H>(s, st.q, k_operand_ptr<H>(ks, sub, lane));
+    floatx16 s[NQB];
+    qk_mfma<H, NQB>(s, st.q, k_operand_ptr<H>(ks, sub, lane));
 
     if constexpr (HAS_MASK) {
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-            const _Float16* mrow = nb == 0 ? mask_row0 : mask_row1;
+        for (int nb = 0; nb < NQB; ++nb) {
+            const _Float16* mrow = mask_row[nb];
             if (mrow != nullptr) {
 #pragma unroll
                 for (int r4 = 0; r4 < 4; ++r4) {
@@ -347,38 +351,39 @@ __device__ __forceinline__ void process_subtile(WaveState<H>& st, const _Float16
         for (int r = 0; r < 16; ++r) {
             const int key = 8 * (r >> 2) + 4 * g + (r & 3);
             if (key >= nvalid) {
-                s[0][r] = -__builtin_inff();
-                s[1][r] = -__builtin_inff();
+#pragma unroll
+                for (int nb = 0; nb < NQB; ++nb) s[nb][r] = -__builtin_inff();
             }
         }
     }
 
-    uint32_t pk[2][8];
-    float ts[2];
-    exp_pack_sum(s, c, st.mc, pk, ts);
-    softmax_check<H>(st, s, c, pk, ts);
-    pv_mfma<H>(st.o, v_operand_ptr<H>(vs, sub, lane), pk);
+    uint32_t pk[NQB][8];
+    float ts[NQB];
+    exp_pack_sum<NQB>(s, c, st.mc, pk, ts);
+    softmax_check<H, NQB>(st, s, c, pk, ts);
+    pv_mfma<H, NQB>(st.o, v_operand_ptr<H>(vs, sub, lane), pk);
 }
 
 // One stage of the software pipeline: three independent pieces of work on three sub-tiles,
 //   s_next = K_{j+1} Q^T          (matrix core)
 //   p_cur  = exp2(s_cur ...)      (vector ALU)
 //   O^T   += V_{j-1}^T p_prev     (matrix core)
-// written out in the order the instructions should issue: the exponentials are cut into 16 chunks
+// written out in the order the instructions should issue: the exponentials are cut into 8 NQB chunks
 // of one fp16 pair (2 fma, 2 exp, 1 pack, 1 dot2: about the duration of one 32x32x16 MFMA), each
 // followed by its share of the matrix instructions, with the LDS operand reads issued PF operands
 // ahead of their use.  A scheduling barrier after every chunk keeps the compiler from regrouping
 // them, so that one wave by itself keeps the matrix core and the vector ALU busy together.
-template <int H>
-__device__ __forceinline__ void pipeline_stage(WaveState<H>& st, floatx16 (&s_next)[2],
-                                               const floatx16 (&s_cur)[2], uint32_t (&p_cur)[2][8],
-                                               const uint32_t (&p_prev)[2][8], const _Float16* krow,
+template <int H, int NQB>
+__device__ __forceinline__ void pipeline_stage(WaveState<H, NQB>& st, floatx16 (&s_next)[NQB],
+                                               const floatx16 (&s_cur)[NQB], uint32_t (&p_cur)[NQB][8],
+                                               const uint32_t (&p_prev)[NQB][8], const _Float16* krow,
                                                const _Float16* vrow, float c) {
     using G = Geometry<H>;
     constexpr int NQK = G::KS;            // operand slots of the first product (K rows)
     constexpr int NPV = 2 * G::DB;        // operand slots of the second product (V^T blocks)
     constexpr int NU = NQK + NPV;
-    constexpr int NM = 2 * NU;            // matrix instructions of this stage
+    constexpr int NM = NQB * NU;          // matrix instructions of this stage
+    constexpr int NC = 8 * NQB;           // chunks of vector work (one fp16 pair each)
     constexpr int D = 2;                  // chunks of vector work issued before the first MFMA
     constexpr int PF = NU < 3 ? NU : 3;   // operand slots fetched ahead
     typedef short short8v __attribute__((ext_vector_type(8)));
@@ -398,7 +403,7 @@ __device__ __forceinline__ void pipeline_stage(WaveState<H>& st, floatx16 (&s_ne
         }
     };
     auto mma = [&](int j) {
-        const int u = j >> 1, nb = j & 1;
+        const int u = j / NQB, nb = j % NQB;
         if (u < NQK) {
             if (u == 0) {
                 floatx16 z;
@@ -418,14 +423,16 @@ __device__ __forceinline__ void pipeline_stage(WaveState<H>& st, floatx16 (&s_ne
     };
 
     const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
-    float ts[2] = {0.f, 0.f};
+    float ts[NQB];
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) ts[nb] = 0.f;
     float e0 = 0.f, e1 = 0.f;   // exponentials of the previous chunk, packed one chunk later
 
 #pragma unroll
     for (int u = 0; u < PF; ++u) fetch(u);
 #pragma unroll
-    for (int i = 0; i <= 16; ++i) {
-        if (i < 16) {
+    for (int i = 0; i <= NC; ++i) {
+        if (i < NC) {
             const int nb = i >> 3, r = (i & 7) * 2;
             const float a0 = __builtin_fmaf(s_cur[nb][r], c, st.mc[nb]);
             const float a1 = __builtin_fmaf(s_cur[nb][r + 1], c, st.mc[nb]);
@@ -441,31 +448,31 @@ __device__ __forceinline__ void pipeline_stage(WaveState<H>& st, floatx16 (&s_ne
             e1 = n1;
         } else {
             const uint32_t pp = pack_rtz(e0, e1);
-            p_cur[1][7] = pp;
-            ts[1] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, pp), ones, ts[1], false);
+            p_cur[NQB - 1][7] = pp;
+            ts[NQB - 1] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, pp), ones, ts[NQB - 1], false);
         }
         if (i >= D) {
-            const int jlo = (i - D) * NM / 16;
-            const int jhi = i == 16 ? NM : (i - D + 1) * NM / 16;
+            const int jlo = (i - D) * NM / NC;
+            const int jhi = i == NC ? NM : (i - D + 1) * NM / NC;
 #pragma unroll
             for (int j = jlo; j < jhi; ++j) {
                 mma(j);
-                if ((j & 1) == 0 && (j >> 1) + PF < NU) fetch((j >> 1) + PF);
+                if (j % NQB == 0 && j / NQB + PF < NU) fetch(j / NQB + PF);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
     }
-    softmax_check<H>(st, s_cur, c, p_cur, ts);
+    softmax_check<H, NQB>(st, s_cur, c, p_cur, ts);
 }
 
-#ifndef FA_WAVES_PER_EU_64
-#define FA_WAVES_PER_EU_64 2
-#endif
-
-template <int H, int NW, int BK, bool HAS_MASK>
-__global__ __launch_bounds__(NW * 64, (H <= 64 ? FA_WAVES_PER_EU_64 : 1)) void fwd_kernel(const FwdParams p) {
+// Template parameters: head_dim H, NW wave64s per workgroup, BK keys per LDS tile, NQB blocks of 32
+// query rows per wave, WPE waves per SIMD the register budget is sized for.
+template <int H, int NW, int BK, int NQB, int WPE, bool HAS_MASK>
+__global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel(const FwdParams p) {
     using G = Geometry<H>;
-    constexpr int BQ = NW * 64;
+    constexpr int QW = 32 * NQB;            // query rows per wave
+    constexpr int BQ = NW * QW;             // query rows per workgroup
+    constexpr int NT = NW * 64;
     constexpr int NSUB = BK / 32;
     static_assert(BK == 64, "the pipelined loop is written for two sub-tiles per tile");
 
@@ -497,17 +504,17 @@ __global__ __launch_bounds__(NW * 64, (H <= 64 ? FA_WAVES_PER_EU_64 : 1)) void f
     const _Float16* kbase = p.k + head_off;
     const _Float16* vbase = p.v + head_off;
     _Float16* obase = p.o + head_off;
-    const int q0 = qt * BQ + wave * 64;
+    const int q0 = qt * BQ + wave * QW;
 
     // V columns beyond H (only when H = 16) stay zero for the whole kernel.
     if constexpr (G::HV != H) {
-        for (int i = tid; i < 2 * VTILE; i += BQ) vs_base[i] = (_Float16)0.f;
+        for (int i = tid; i < 2 * VTILE; i += NT) vs_base[i] = (_Float16)0.f;
         __syncthreads();
     }
 
-    WaveState<H> st;
+    WaveState<H, NQB> st;
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int nb = 0; nb < NQB; ++nb) {
         const int row = q0 + nb * 32 + ln;
 #pragma unroll
         for (int kk = 0; kk < G::KS; ++kk) {
@@ -533,11 +540,13 @@ __global__ __launch_bounds__(NW * 64, (H <= 64 ? FA_WAVES_PER_EU_64 : 1)) void f
 
     if constexpr (HAS_MASK) {
         // Additive-mask variant: plain double-buffered loop, one sub-tile after the other.
-        const _Float16* mask_row0 = nullptr;
-        const _Float16* mask_row1 = nullptr;
+        const _Float16* mask_row[NQB];
         const _Float16* mb = p.mask + (int64_t)b * L * L;
-        if (q0 + ln < L) mask_row0 = mb + (int64_t)(q0 + ln) * L;
-        if (q0 + 32 + ln < L) mask_row1 = mb + (int64_t)(q0 + 32 + ln) * L;
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb) {
+            const int row = q0 + nb * 32 + ln;
+            mask_row[nb] = row < L ? mb + (int64_t)row * L : nullptr;
+        }
 
         loader.load_k(kbase, sl, 0, L, tid);
         loader.load_v(vbase, sl, 0, L, tid);
@@ -555,9 +564,8 @@ __global__ __launch_bounds__(NW * 64, (H <= 64 ? FA_WAVES_PER_EU_64 : 1)) void f
             for (int sub = 0; sub < NSUB; ++sub) {
                 const int nvalid = L - t * BK - sub * 32;
                 if (nvalid > 0)
-                    process_subtile<H, true, true>(st, ks_base + buf * KTILE, vs_base + buf * VTILE, sub,
-                                                   nvalid, c, lane, mask_row0, mask_row1,
-                                                   t * BK + sub * 32, L);
+                    process_subtile<H, NQB, true, true>(st, ks_base + buf * KTILE, vs_base + buf * VTILE,
+                                                        sub, nvalid, c, lane, mask_row, t * BK + sub * 32, L);
             }
             if (has_next) {
                 loader.store_k(ks_base + (buf ^ 1) * KTILE, tid);
@@ -580,14 +588,14 @@ __global__ __launch_bounds__(NW * 64, (H <= 64 ? FA_WAVES_PER_EU_64 : 1)) void f
 
         const bool ragged = nfull < ntiles;
         if (nfull > 0) {
-            floatx16 sa[2], sb[2];
-            uint32_t pa[2][8], pb[2][8];
-            float ts[2];
+            floatx16 sa[NQB], sb[NQB];
+            uint32_t pa[NQB][8], pb[NQB][8];
+            float ts[NQB];
             // stage 0 (no PV yet)
-            qk_mfma<H>(sa, st.q, k_operand_ptr<H>(ks_base, 0, lane));
-            qk_mfma<H>(sb, st.q, k_operand_ptr<H>(ks_base, 1, lane));
-            exp_pack_sum(sa, c, st.mc, pa, ts);
-            softmax_check<H>(st, sa, c, pa, ts);
+            qk_mfma<H, NQB>(sa, st.q, k_operand_ptr<H>(ks_base, 0, lane));
+            qk_mfma<H, NQB>(sb, st.q, k_operand_ptr<H>(ks_base, 1, lane));
+            exp_pack_sum<NQB>(sa, c, st.mc, pa, ts);
+            softmax_check<H, NQB>(st, sa, c, pa, ts);
             // every wave is done with K tile 0 before anyone overwrites its buffer
             __syncthreads();
 
@@ -596,23 +604,23 @@ __global__ __launch_bounds__(NW * 64, (H <= 64 ? FA_WAVES_PER_EU_64 : 1)) void f
                 const _Float16* vcur = vs_base + (T & 1) * VTILE;
                 loader.load_k(kbase, sl, (T + 2) * BK, L, tid);
                 loader.load_v(vbase, sl, (T + 1) * BK, L, tid);
-                pipeline_stage<H>(st, sa, sb, pb, pa, k_operand_ptr<H>(kcur, 0, lane),
-                                  v_operand_ptr<H>(vcur, 0, lane), c);
-                pipeline_stage<H>(st, sb, sa, pa, pb, k_operand_ptr<H>(kcur, 1, lane),
-                                  v_operand_ptr<H>(vcur, 1, lane), c);
+                pipeline_stage<H, NQB>(st, sa, sb, pb, pa, k_operand_ptr<H>(kcur, 0, lane),
+                                       v_operand_ptr<H>(vcur, 0, lane), c);
+                pipeline_stage<H, NQB>(st, sb, sa, pa, pb, k_operand_ptr<H>(kcur, 1, lane),
+                                       v_operand_ptr<H>(vcur, 1, lane), c);
                 loader.store_k(ks_base + (T & 1) * KTILE, tid);
                 loader.store_v(vs_base + ((T + 1) & 1) * VTILE, tid);
                 __syncthreads();
             }
 
             // drain: exponentials of the last full sub-tile, PV of the last two
+            // (PV of sub-tile j - 1 goes first: a rescale triggered by sub-tile j must see it in O)
             const _Float16* vlast = vs_base + ((nfull - 1) & 1) * VTILE;
             if (ragged) loader.load_v(vbase, sl, nfull * BK, L, tid);
-            // (PV of sub-tile j - 1 goes first: a rescale triggered by sub-tile j must see it in O)
-            pv_mfma<H>(st.o, v_operand_ptr<H>(vlast, 0, lane), pa);
-            exp_pack_sum(sb, c, st.mc, pb, ts);
-            softmax_check<H>(st, sb, c, pb, ts);
-            pv_mfma<H>(st.o, v_operand_ptr<H>(vlast, 1, lane), pb);
+            pv_mfma<H, NQB>(st.o, v_operand_ptr<H>(vlast, 0, lane), pa);
+            exp_pack_sum<NQB>(sb, c, st.mc, pb, ts);
+            softmax_check<H, NQB>(st, sb, c, pb, ts);
+            pv_mfma<H, NQB>(st.o, v_operand_ptr<H>(vlast, 1, lane), pb);
             if (ragged) {
                 loader.store_v(vs_base + (nfull & 1) * VTILE, tid);
                 __syncthreads();
@@ -621,19 +629,20 @@ __global__ __launch_bounds__(NW * 64, (H <= 64 ? FA_WAVES_PER_EU_64 : 1)) void f
         if (ragged) {
             const int buf = nfull & 1;
             const int key0 = nfull * BK;
+            const _Float16* no_mask[NQB] = {};
 #pragma unroll
             for (int sub = 0; sub < NSUB; ++sub) {
                 const int nvalid = L - key0 - sub * 32;
                 if (nvalid > 0)
-                    process_subtile<H, true, false>(st, ks_base + buf * KTILE, vs_base + buf * VTILE, sub,
-                                                    nvalid, c, lane, nullptr, nullptr, key0 + sub * 32, L);
+                    process_subtile<H, NQB, true, false>(st, ks_base + buf * KTILE, vs_base + buf * VTILE,
+                                                         sub, nvalid, c, lane, no_mask, key0 + sub * 32, L);
             }
         }
     }
 
     // ---- epilogue: O = O^T / l, f16, 8-byte stores ------------------------------------------
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int nb = 0; nb < NQB; ++nb) {
         const float lt = pair_sum(st.l[nb]);
         // A row whose every key carried a -inf mask has l = 0: emit zeros rather than NaN.
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
