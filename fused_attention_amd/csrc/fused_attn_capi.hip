@@ -22,13 +22,15 @@ struct Shape {
 };
 
 // Three shapes, picked by how many workgroups the problem gives the 256 compute units:
-//   {8, 2}  eight 64-row waves share one K/V stream between 512 queries: best once every compute
-//           unit still gets two such workgroups (head_dim <= 64, two waves per SIMD);
+//   {8, 2}  eight 64-row waves share one K/V stream between 512 queries (head_dim <= 64, two
+//           waves per SIMD), run by the ping-pong kernel: best once every compute unit still gets
+//           two such workgroups; the additive-mask variant uses the plain eight-wave kernel;
 //   {4, 2}  four 64-row waves, 256 queries per workgroup;
 //   {4, 1}  four 32-row waves, 128 queries per workgroup, three (head_dim <= 64) or two
 //           (head_dim 128) waves per SIMD: more, smaller workgroups for short sequences.
 // head_dim 128 with 64-row waves needs the whole register file of a SIMD for one wave.
 Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask) {
+
     // the additive-mask variant at head_dim 128 only exists with 32-row waves (register budget)
     if (H > 64 && has_mask) return {4, 1};
     const int64_t wgs512 = B * R * ((L + 511) / 512);
@@ -57,6 +59,24 @@ hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
+template <int H, int NW, int NQB, int WPE>
+hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
+    constexpr int lds = fa::lds_bytes_pingpong<H, NQB>();
+    auto kernel = fa::fwd_kernel_pingpong<H, NW, NQB, WPE>;
+    if constexpr (lds > 64 * 1024) {
+        static std::once_flag once;
+        static hipError_t attr_status = hipSuccess;
+        std::call_once(once, [&] {
+            attr_status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        });
+        if (attr_status != hipSuccess) return attr_status;
+    }
+    const int grid = p.wgs_per_xcd * fa::kNumXcd;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * 64), lds, stream, p);
+    return hipGetLastError();
+}
+
 template <int H, bool HAS_MASK>
 hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) {
     if constexpr (H > 64) {
@@ -65,7 +85,12 @@ hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) 
         else
             return sh.nqb == 2 ? launch<H, 4, 2, 1, false>(p, stream) : launch<H, 4, 1, 2, false>(p, stream);
     } else {
-        if (sh.waves == 8) return launch<H, 8, 2, 2, HAS_MASK>(p, stream);
+        if (sh.waves == 8) {
+            if constexpr (HAS_MASK)
+                return launch<H, 8, 2, 2, true>(p, stream);
+            else
+                return launch_pingpong<H, 8, 2, 2>(p, stream);
+        }
         return sh.nqb == 2 ? launch<H, 4, 2, 2, HAS_MASK>(p, stream) : launch<H, 4, 1, 3, HAS_MASK>(p, stream);
     }
 }

@@ -115,16 +115,18 @@ struct TileLoader {
     u32x4 kreg[NP];
     u32x4 vreg[NP];
 
+    // Rows at or beyond L are read from row L - 1 instead of being predicated off (a predicated
+    // load into a zeroed register makes every load wait for the one before it).  Such keys are
+    // masked to -inf before the softmax, and a probability of exactly zero times a finite V row
+    // contributes nothing.
     static __device__ __forceinline__ void load(u32x4 (&reg)[NP], const _Float16* base, int64_t stride_l,
                                                 int key0, int L, int tid) {
+        if (key0 >= L) return;
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
-            const int idx = tid + i * NT;
-            const int key = key0 + idx / CPR;
-            u32x4 x = {0u, 0u, 0u, 0u};   // rows past the end of the sequence read as zeros
-            if ((EXACT || idx < NCHUNK) && key < L)
-                x = *reinterpret_cast<const u32x4*>(base + (int64_t)key * stride_l + (idx % CPR) * 8);
-            reg[i] = x;
+            const int idx = EXACT ? tid + i * NT : min(tid + i * NT, NCHUNK - 1);
+            const int key = min(key0 + idx / CPR, L - 1);
+            reg[i] = *reinterpret_cast<const u32x4*>(base + (int64_t)key * stride_l + (idx % CPR) * 8);
         }
     }
     template <int STR>
@@ -465,6 +467,38 @@ __device__ __forceinline__ void pipeline_stage(WaveState<H, NQB>& st, floatx16 (
     softmax_check<H, NQB>(st, s_cur, c, p_cur, ts);
 }
 
+// O = O^T / l in f32, one rounding to fp16, 8-byte stores of four consecutive head-dim elements.
+template <int H, int NQB>
+__device__ __forceinline__ void store_output(WaveState<H, NQB>& st, _Float16* obase, int64_t stride_l,
+                                             int q0, int L, int lane) {
+    using G = Geometry<H>;
+    const int g = lane >> 5;
+    const int ln = lane & 31;
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) {
+        const float lt = pair_sum(st.l[nb]);
+        // A row whose every key carried a -inf mask has l = 0: emit zeros rather than NaN.
+        const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+        const int row = q0 + nb * 32 + ln;
+        if (row < L) {
+            _Float16* orow = obase + (int64_t)row * stride_l;
+#pragma unroll
+            for (int db = 0; db < G::DB; ++db) {
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    const int d = db * 32 + 8 * r4 + 4 * g;
+                    if (G::HV == H || d < H) {
+                        half4 hv;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) hv[j] = (_Float16)(st.o[db][nb][4 * r4 + j] * inv);
+                        *reinterpret_cast<u32x2*>(orow + d) = __builtin_bit_cast(u32x2, hv);
+                    }
+                }
+            }
+        }
+    }
+}
+
 // Template parameters: head_dim H, NW wave64s per workgroup, BK keys per LDS tile, NQB blocks of 32
 // query rows per wave, WPE waves per SIMD the register budget is sized for.
 template <int H, int NW, int BK, int NQB, int WPE, bool HAS_MASK>
@@ -640,30 +674,262 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel(const FwdParams p) {
         }
     }
 
-    // ---- epilogue: O = O^T / l, f16, 8-byte stores ------------------------------------------
+    store_output<H, NQB>(st, obase, p.stride_l, q0, L, lane);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Ping-pong variant: eight waves per workgroup, two per SIMD.  On this hardware a wave does not
+// overlap its own vector work with its own matrix instructions, so the overlap has to come from
+// the two waves that share a SIMD.  The waves form two groups (0-3 and 4-7, one wave of each per
+// SIMD) that alternate between a vector phase (exponentials of sub-tile j) and a matrix phase
+// (PV of sub-tile j, QK^T of sub-tile j + 1), the second group one phase behind the first, with a
+// workgroup barrier between phases: while one group keeps the matrix cores busy the other does
+// the softmax on the vector ALUs of the same SIMDs.
+//
+// K and V stream through three-slot LDS rings.  Group 0 loads K, group 1 loads V, each during its
+// own vector phases: at its first vector phase of tile T a group writes tile T + 2 (fetched into
+// registers one tile earlier) to the ring and, at the start of the following matrix phase, issues
+// the global loads of tile T + 3.  Slot (T + 2) % 3 last held tile T - 1, whose final reader
+// finished at least one barrier earlier.
+template <int H, int NQB>
+constexpr int lds_bytes_pingpong() {
+    using G = Geometry<H>;
+    return 3 * 64 * (G::KSTR + G::VSTR) * (int)sizeof(_Float16);
+}
+
+__device__ __forceinline__ void phase_barrier() {
+    // LDS traffic of this wave is complete (writes visible, reads returned) before the barrier;
+    // global loads in flight are deliberately not waited for.  The scheduling barriers keep the
+    // compiler from moving matrix or vector instructions of one phase into the next.
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// One group's share of a 64-key tile: per-thread chunk offsets are computed once, a tile is then
+// fetched with one pointer bump and NP 16-byte loads.
+template <int H, int NT>
+struct GroupLoader {
+    static constexpr int CPR = H / 8;
+    static constexpr int NCHUNK = 64 * CPR;
+    static constexpr int NP = (NCHUNK + NT - 1) / NT;
+    static constexpr bool EXACT = NCHUNK % NT == 0;
+    u32x4 reg[NP];
+    int64_t goff[NP];   // element offset of the chunk inside a tile
+    int loff[NP];       // element offset of the chunk inside an LDS tile
+    int row[NP];
+    int col[NP];
+
+    __device__ __forceinline__ void init(int64_t stride_l, int lds_stride, int gtid) {
 #pragma unroll
-    for (int nb = 0; nb < NQB; ++nb) {
-        const float lt = pair_sum(st.l[nb]);
-        // A row whose every key carried a -inf mask has l = 0: emit zeros rather than NaN.
-        const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-        const int row = q0 + nb * 32 + ln;
-        if (row < L) {
-            _Float16* orow = obase + (int64_t)row * p.stride_l;
+        for (int i = 0; i < NP; ++i) {
+            const int idx = gtid + i * NT;
+            row[i] = (EXACT || idx < NCHUNK) ? idx / CPR : (1 << 30);
+            col[i] = (idx % CPR) * 8;
+            goff[i] = (int64_t)(idx / CPR) * stride_l + (idx % CPR) * 8;
+            loff[i] = (idx / CPR) * lds_stride + (idx % CPR) * 8;
+        }
+    }
+    // Rows at or beyond L are read from row L - 1 instead (no predicated loads, so no load ever
+    // waits for another): their scores are masked to -inf, or belong to sub-tiles that are never
+    // consumed, and a probability of exactly zero times a finite V row contributes nothing.
+    __device__ __forceinline__ void load(const _Float16* src, int64_t stride_l, int key0, int L) {
+        if (key0 >= L) return;
+        if (key0 + 64 <= L && EXACT) {
+            const _Float16* tile = src + (int64_t)key0 * stride_l;
 #pragma unroll
-            for (int db = 0; db < G::DB; ++db) {
+            for (int i = 0; i < NP; ++i) reg[i] = *reinterpret_cast<const u32x4*>(tile + goff[i]);
+        } else {
 #pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    const int d = db * 32 + 8 * r4 + 4 * g;
-                    if (G::HV == H || d < H) {
-                        half4 hv;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) hv[j] = (_Float16)(st.o[db][nb][4 * r4 + j] * inv);
-                        *reinterpret_cast<u32x2*>(orow + d) = __builtin_bit_cast(u32x2, hv);
-                    }
-                }
+            for (int i = 0; i < NP; ++i) {
+                const int r = min(key0 + min(row[i], 63), L - 1);
+                reg[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)r * stride_l + col[i]);
             }
         }
     }
+    __device__ __forceinline__ void store(_Float16* dst) const {
+#pragma unroll
+        for (int i = 0; i < NP; ++i)
+            if (EXACT || row[i] < 64) *reinterpret_cast<u32x4*>(dst + loff[i]) = reg[i];
+    }
+};
+
+template <int H, int NW, int NQB, int WPE>
+__global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdParams p) {
+    using G = Geometry<H>;
+    constexpr int BK = 64;
+    static_assert(NW == 8 || NW == 16, "two groups of four or eight waves");
+    constexpr int QW = 32 * NQB;
+    constexpr int BQ = NW * QW;
+    constexpr int KTILE = BK * G::KSTR;
+    constexpr int VTILE = BK * G::VSTR;
+    constexpr int GT = NW * 32;             // threads of one group
+    typedef short short8v __attribute__((ext_vector_type(8)));
+
+    extern __shared__ __attribute__((aligned(16))) _Float16 smem[];
+    _Float16* const ks_base = smem;                      // [3][BK][KSTR]
+    _Float16* const vs_base = smem + 3 * KTILE;          // [3][BK][VSTR]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // waves w, w + 4, w + 8, ... share a SIMD: group = bit 2 of the wave index
+    const int grp = (wave >> 2) & 1;
+    const int gtid = ((wave >> 3) << 8) | (tid & 255);
+    const int g = lane >> 5;
+    const int ln = lane & 31;
+
+    const int wg = blockIdx.x;
+    const int logical = (wg % kNumXcd) * p.wgs_per_xcd + wg / kNumXcd;
+    if (logical >= p.total_wgs) return;
+    const int bh = logical / p.n_qtiles;
+    const int qt = logical % p.n_qtiles;
+    const int b = bh / p.R;
+    const int h = bh % p.R;
+    const int L = p.L;
+
+    const int64_t head_off = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h;
+    const _Float16* qbase = p.q + head_off;
+    const _Float16* kbase = p.k + head_off;
+    const _Float16* vbase = p.v + head_off;
+    _Float16* obase = p.o + head_off;
+    const int q0 = qt * BQ + wave * QW;
+    const int64_t sl = p.stride_l;
+
+    if constexpr (G::HV != H) {
+        for (int i = tid; i < 3 * VTILE; i += NW * 64) vs_base[i] = (_Float16)0.f;
+        __syncthreads();
+    }
+
+    WaveState<H, NQB> st;
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) {
+        const int row = q0 + nb * 32 + ln;
+#pragma unroll
+        for (int kk = 0; kk < G::KS; ++kk) {
+            u32x4 w = {0u, 0u, 0u, 0u};
+            if (row < L)
+                w = *reinterpret_cast<const u32x4*>(qbase + (int64_t)row * sl + kk * 16 + 8 * g);
+            st.q[nb][kk] = __builtin_bit_cast(half8, w);
+        }
+        st.m[nb] = -__builtin_inff();
+        st.mc[nb] = __builtin_inff();
+        st.l[nb] = 0.f;
+#pragma unroll
+        for (int db = 0; db < G::DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) st.o[db][nb][r] = 0.f;
+    }
+
+    const float c = p.scale_log2e;
+    const int nsub = (L + 31) >> 5;
+    const int last_valid = L - (nsub - 1) * 32;     // valid keys in the last sub-tile (1..32)
+
+    // Group 0 streams K, group 1 streams V.
+    GroupLoader<H, GT> gl;
+    gl.init(sl, grp == 0 ? G::KSTR : G::VSTR, gtid);
+    const _Float16* const gsrc = grp == 0 ? kbase : vbase;
+    _Float16* const ring = grp == 0 ? ks_base : vs_base;
+    const int ring_tile = grp == 0 ? KTILE : VTILE;
+
+    // prologue: tiles 0 and 1 into the ring, tile 2 into registers
+    gl.load(gsrc, sl, 0, L);
+    gl.store(ring);
+    gl.load(gsrc, sl, BK, L);
+    gl.store(ring + ring_tile);
+    gl.load(gsrc, sl, 2 * BK, L);
+    __syncthreads();
+
+    floatx16 s[NQB];
+    uint32_t pk[NQB][8];
+    float ts[NQB];
+    qk_mfma<H, NQB>(s, st.q, k_operand_ptr<H>(ks_base, 0, lane));
+    if (grp == 1) phase_barrier();                  // the second group runs one phase behind
+
+    for (int j = 0; j < nsub; ++j) {
+        const int T = j >> 1;
+        const int jn = j + 1;
+        // ---- vector phase -------------------------------------------------------------------
+        // First the LDS traffic of this phase: the tile fetched one tile-time ago goes into the
+        // ring, and the K rows of the next sub-tile come out of it (they were written several
+        // phases ago), so that the matrix phase starts with its operands in registers.
+        if ((j & 1) == 0) gl.store(ring + ((T + 2) % 3) * ring_tile);
+        half8 kop[G::KS];
+        {
+            const _Float16* krow = k_operand_ptr<H>(ks_base + ((jn >> 1) % 3) * KTILE, jn & 1, lane);
+#pragma unroll
+            for (int kk = 0; kk < G::KS; ++kk) kop[kk] = *reinterpret_cast<const half8*>(krow + kk * 16);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (j == nsub - 1 && last_valid < 32) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+                if (key >= last_valid) {
+#pragma unroll
+                    for (int nb = 0; nb < NQB; ++nb) s[nb][r] = -__builtin_inff();
+                }
+            }
+        }
+        exp_pack_sum<NQB>(s, c, st.mc, pk, ts);
+        softmax_check<H, NQB>(st, s, c, pk, ts);
+        phase_barrier();
+        // ---- matrix phase -------------------------------------------------------------------
+        const _Float16* vrow = v_operand_ptr<H>(vs_base + (T % 3) * VTILE, j & 1, lane);
+        half8 vop[2][G::DB];
+        auto vfetch = [&](int t) {
+#pragma unroll
+            for (int db = 0; db < G::DB; ++db) {
+                const _Float16* p0 = vrow + (16 * t) * G::VSTR + db * 32;
+                const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS short4v*)(p0));
+                const short4v hi =
+                    __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS short4v*)(p0 + 8 * G::VSTR));
+                const short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                vop[t][db] = __builtin_bit_cast(half8, both);
+            }
+        };
+        vfetch(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < G::KS; ++kk) {
+#pragma unroll
+            for (int nb = 0; nb < NQB; ++nb) {
+                if (kk == 0) {
+                    floatx16 z;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) z[r] = 0.f;
+                    s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kop[kk], st.q[nb][kk], z, 0, 0, 0);
+                } else {
+                    s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kop[kk], st.q[nb][kk], s[nb], 0, 0, 0);
+                }
+            }
+            if (kk == 0) {
+                vfetch(1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int db = 0; db < G::DB; ++db) {
+#pragma unroll
+                for (int nb = 0; nb < NQB; ++nb) {
+                    const u32x4 w = {pk[nb][4 * t], pk[nb][4 * t + 1], pk[nb][4 * t + 2], pk[nb][4 * t + 3]};
+                    st.o[db][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                        vop[t][db], __builtin_bit_cast(half8, w), st.o[db][nb], 0, 0, 0);
+                }
+            }
+        }
+        // the global loads of the tile three ahead go last: they cost this wave a few issue slots
+        // while its matrix instructions are already queued
+        if ((j & 1) == 0) gl.load(gsrc, sl, (T + 3) * BK, L);
+        phase_barrier();
+    }
+    if (grp == 0) phase_barrier();
+
+    store_output<H, NQB>(st, obase, sl, q0, L, lane);
 }
 
 }  // namespace fa
