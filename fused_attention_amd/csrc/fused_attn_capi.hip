@@ -35,7 +35,7 @@ Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask) {
     if (H > 64 && has_mask) return {4, 1};
     const int64_t wgs512 = B * R * ((L + 511) / 512);
     const int64_t wgs256 = B * R * ((L + 255) / 256);
-    if (H > 64) return wgs256 >= 6 * kNumCu ? Shape{4, 2} : Shape{4, 1};
+    if (H > 64) return wgs256 >= 2 * kNumCu ? Shape{8, 1} : Shape{4, 1};
     if (wgs512 >= 2 * kNumCu) return {8, 2};
     return wgs256 >= 2 * kNumCu ? Shape{4, 2} : Shape{4, 1};
 }
@@ -82,6 +82,8 @@ hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) 
     if constexpr (H > 64) {
         if constexpr (HAS_MASK)
             return launch<H, 4, 1, 2, true>(p, stream);
+        else if (sh.waves == 8)
+            return launch_pingpong<H, 8, 1, 2>(p, stream);
         else
             return sh.nqb == 2 ? launch<H, 4, 2, 1, false>(p, stream) : launch<H, 4, 1, 2, false>(p, stream);
     } else {

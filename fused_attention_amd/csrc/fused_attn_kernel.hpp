@@ -861,21 +861,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
 #pragma unroll
             for (int kk = 0; kk < G::KS; ++kk) kop[kk] = *reinterpret_cast<const half8*>(krow + kk * 16);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        if (j == nsub - 1 && last_valid < 32) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int key = 8 * (r >> 2) + 4 * g + (r & 3);
-                if (key >= last_valid) {
-#pragma unroll
-                    for (int nb = 0; nb < NQB; ++nb) s[nb][r] = -__builtin_inff();
-                }
-            }
-        }
-        exp_pack_sum<NQB>(s, c, st.mc, pk, ts);
-        softmax_check<H, NQB>(st, s, c, pk, ts);
-        phase_barrier();
-        // ---- matrix phase -------------------------------------------------------------------
+        // ... and the first half of the V^T operands of this sub-tile
         const _Float16* vrow = v_operand_ptr<H>(vs_base + (T % 3) * VTILE, j & 1, lane);
         half8 vop[2][G::DB];
         auto vfetch = [&](int t) {
@@ -891,6 +877,20 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
         };
         vfetch(0);
         __builtin_amdgcn_sched_barrier(0);
+        if (j == nsub - 1 && last_valid < 32) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+                if (key >= last_valid) {
+#pragma unroll
+                    for (int nb = 0; nb < NQB; ++nb) s[nb][r] = -__builtin_inff();
+                }
+            }
+        }
+        exp_pack_sum<NQB>(s, c, st.mc, pk, ts);
+        softmax_check<H, NQB>(st, s, c, pk, ts);
+        phase_barrier();
+        // ---- matrix phase -------------------------------------------------------------------
 #pragma unroll
         for (int kk = 0; kk < G::KS; ++kk) {
 #pragma unroll
