@@ -11,7 +11,8 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libfused_attn_gfx950.so")
 
 # every symbol include/fused_attn.h declares
-EXPORTS = ("fa_fwd", "fa_fwd_query", "fa_strerror", "fa_fwd_timed")
+EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_query", "fa_strerror", "fa_fwd_timed")
+FLAG_CAUSAL = 1
 
 _lib = None
 
@@ -38,6 +39,9 @@ def load_library():
     fwd_args = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, f32, vp]
     lib.fa_fwd.argtypes = fwd_args
     lib.fa_fwd.restype = ctypes.c_int
+    lib.fa_fwd_ex.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, f32,
+                              ctypes.c_int, vp]
+    lib.fa_fwd_ex.restype = ctypes.c_int
     lib.fa_fwd_timed.argtypes = fwd_args + [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
     lib.fa_fwd_timed.restype = ctypes.c_int
     lib.fa_fwd_query.argtypes = [i64]
@@ -81,11 +85,13 @@ def _current_stream(q):
     return torch.cuda.current_stream(q.device).cuda_stream
 
 
-def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None):
-    """Runs fa_fwd on torch GPU tensors (fp16, contiguous) on torch's current stream.
+def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None, causal=False,
+            return_lse=False):
+    """Runs fa_fwd_ex on torch GPU tensors (fp16, contiguous) on torch's current stream.
 
     layout 'blf' takes [B, L, R*head_dim] tensors, 'bhld' takes [B, R, L, head_dim] tensors.
-    Returns `out` (allocated like q when not given).
+    causal=True restricts query i to keys j <= i.  Returns `out` (allocated like q when not
+    given), or (out, lse) with lse a float32 [B, R, L] tensor when return_lse is set.
     """
     import torch
 
@@ -94,12 +100,14 @@ def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None):
         out = torch.empty_like(q)
     if scale is None:
         scale = 1.0 / math.sqrt(head_dim)
+    lse = torch.empty((B, R, L), dtype=torch.float32, device=q.device) if return_lse else None
     with torch.cuda.device(q.device):
-        status = fwd_raw(q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                         mask.data_ptr() if mask is not None else 0, out.data_ptr(),
-                         B, R, L, head_dim, sb, sh, sl, scale, _current_stream(q))
+        status = load_library().fa_fwd_ex(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr() if mask is not None else None,
+            out.data_ptr(), lse.data_ptr() if lse is not None else None, B, R, L, head_dim, sb, sh, sl,
+            scale, FLAG_CAUSAL if causal else 0, _current_stream(q) or None)
     _check(status)
-    return out
+    return (out, lse) if return_lse else out
 
 
 def forward_timed(q, k, v, head_dim, out, iters, mask=None, layout="blf", scale=None):

@@ -7,6 +7,8 @@
 #include "../../include/fused_attn.h"
 
 #include <mutex>
+#include <utility>
+#include <vector>
 
 namespace {
 
@@ -40,19 +42,29 @@ Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask) {
     return wgs256 >= 2 * kNumCu ? Shape{4, 2} : Shape{4, 1};
 }
 
-template <int H, int NW, int NQB, int WPE, bool HAS_MASK>
+// Dynamic LDS above 64 KiB has to be opted into per kernel function and per device: done on the
+// first launch of that kernel on that device.
+hipError_t allow_large_lds(const void* kernel, int bytes) {
+    static std::mutex lock;
+    static std::vector<std::pair<const void*, int>> done;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> guard(lock);
+    for (const auto& d : done)
+        if (d.first == kernel && d.second == dev) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done.emplace_back(kernel, dev);
+    return e;
+}
+
+template <int H, int NW, int NQB, int WPE, int MODE>
 hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
     constexpr int lds = fa::lds_bytes<H, NW, kKeyTile>();
-    auto kernel = fa::fwd_kernel<H, NW, kKeyTile, NQB, WPE, HAS_MASK>;
-    // Dynamic LDS above 64 KiB has to be opted into once per kernel function.
+    auto kernel = fa::fwd_kernel<H, NW, kKeyTile, NQB, WPE, MODE>;
     if constexpr (lds > 64 * 1024) {
-        static std::once_flag once;
-        static hipError_t attr_status = hipSuccess;
-        std::call_once(once, [&] {
-            attr_status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        });
-        if (attr_status != hipSuccess) return attr_status;
+        const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), lds);
+        if (e != hipSuccess) return e;
     }
     const int grid = p.wgs_per_xcd * fa::kNumXcd;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * 64), lds, stream, p);
@@ -64,46 +76,38 @@ hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
     constexpr int lds = fa::lds_bytes_pingpong<H, NQB>();
     auto kernel = fa::fwd_kernel_pingpong<H, NW, NQB, WPE>;
     if constexpr (lds > 64 * 1024) {
-        static std::once_flag once;
-        static hipError_t attr_status = hipSuccess;
-        std::call_once(once, [&] {
-            attr_status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        });
-        if (attr_status != hipSuccess) return attr_status;
+        const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), lds);
+        if (e != hipSuccess) return e;
     }
     const int grid = p.wgs_per_xcd * fa::kNumXcd;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * 64), lds, stream, p);
     return hipGetLastError();
 }
 
-template <int H, bool HAS_MASK>
+template <int H, int MODE>
 hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) {
-    if constexpr (H > 64) {
-        if constexpr (HAS_MASK)
-            return launch<H, 4, 1, 2, true>(p, stream);
-        else if (sh.waves == 8)
-            return launch_pingpong<H, 8, 1, 2>(p, stream);
+    if constexpr (MODE != fa::kPlain) {
+        // masked variants: four waves, 64-row waves where the registers allow it
+        if constexpr (H > 64)
+            return launch<H, 4, 1, 2, MODE>(p, stream);
         else
-            return sh.nqb == 2 ? launch<H, 4, 2, 1, false>(p, stream) : launch<H, 4, 1, 2, false>(p, stream);
+            return sh.nqb == 2 ? launch<H, 4, 2, 2, MODE>(p, stream) : launch<H, 4, 1, 3, MODE>(p, stream);
+    } else if constexpr (H > 64) {
+        if (sh.waves == 8) return launch_pingpong<H, 8, 1, 2>(p, stream);
+        return sh.nqb == 2 ? launch<H, 4, 2, 1, MODE>(p, stream) : launch<H, 4, 1, 2, MODE>(p, stream);
     } else {
-        if (sh.waves == 8) {
-            if constexpr (HAS_MASK)
-                return launch<H, 8, 2, 2, true>(p, stream);
-            else
-                return launch_pingpong<H, 8, 2, 2>(p, stream);
-        }
-        return sh.nqb == 2 ? launch<H, 4, 2, 2, HAS_MASK>(p, stream) : launch<H, 4, 1, 3, HAS_MASK>(p, stream);
+        if (sh.waves == 8) return launch_pingpong<H, 8, 2, 2>(p, stream);
+        return sh.nqb == 2 ? launch<H, 4, 2, 2, MODE>(p, stream) : launch<H, 4, 1, 3, MODE>(p, stream);
     }
 }
 
-template <bool HAS_MASK>
+template <int MODE>
 hipError_t dispatch(int64_t H, Shape sh, const fa::FwdParams& p, hipStream_t stream) {
     switch (H) {
-        case 16: return dispatch_shape<16, HAS_MASK>(sh, p, stream);
-        case 32: return dispatch_shape<32, HAS_MASK>(sh, p, stream);
-        case 64: return dispatch_shape<64, HAS_MASK>(sh, p, stream);
-        case 128: return dispatch_shape<128, HAS_MASK>(sh, p, stream);
+        case 16: return dispatch_shape<16, MODE>(sh, p, stream);
+        case 32: return dispatch_shape<32, MODE>(sh, p, stream);
+        case 64: return dispatch_shape<64, MODE>(sh, p, stream);
+        case 128: return dispatch_shape<128, MODE>(sh, p, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -112,7 +116,7 @@ bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u
 
 int validate(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,
              int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h, int64_t stride_l,
-             fa::FwdParams* p, float scale, Shape* shape) {
+             fa::FwdParams* p, float scale, Shape* shape, bool causal, void* lse) {
     if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return FA_ERR_NULL_POINTER;
     if (!fa_fwd_query(H)) return FA_ERR_BAD_HEAD_DIM;
     if (B < 1 || R < 1 || L < 1) return FA_ERR_BAD_SHAPE;
@@ -122,7 +126,7 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     if (mask != nullptr && (reinterpret_cast<uintptr_t>(mask) & 1u) != 0) return FA_ERR_MISALIGNED;
     constexpr int64_t kMaxInt = 0x7fffffff;
     if (L > kMaxInt - 4096 || B > kMaxInt || R > kMaxInt) return FA_ERR_TOO_LARGE;
-    *shape = pick_shape(B, R, L, H, mask != nullptr);
+    *shape = pick_shape(B, R, L, H, mask != nullptr || causal);
     const int64_t bq = shape->rows();
     const int64_t n_qtiles = (L + bq - 1) / bq;
     const int64_t total = B * R * n_qtiles;
@@ -137,6 +141,7 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     p->v = static_cast<const _Float16*>(v);
     p->mask = static_cast<const _Float16*>(mask);
     p->o = static_cast<_Float16*>(out);
+    p->lse = static_cast<float*>(lse);
     p->stride_b = stride_b;
     p->stride_h = stride_h;
     p->stride_l = stride_l;
@@ -166,22 +171,41 @@ const char* fa_strerror(int status) {
             return "fa_fwd: strides must be non-negative multiples of 8 elements and stride_l >= head_dim";
         case FA_ERR_MISALIGNED: return "fa_fwd: q, k, v and out must be 16-byte aligned";
         case FA_ERR_TOO_LARGE: return "fa_fwd: problem size exceeds the supported index range";
+        case FA_ERR_BAD_FLAGS: return "fa_fwd_ex: unknown flag, or FA_FLAG_CAUSAL together with a mask";
         default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
     return "fa_fwd: unknown status";
 }
 
+int fa_fwd_ex(const void* q, const void* k, const void* v, const void* mask, void* out, void* lse,
+              int64_t B, int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h,
+              int64_t stride_l, float scale, int flags, void* stream) {
+    if ((flags & ~FA_FLAG_CAUSAL) != 0) return FA_ERR_BAD_FLAGS;
+    const bool causal = (flags & FA_FLAG_CAUSAL) != 0;
+    if (causal && mask != nullptr) return FA_ERR_BAD_FLAGS;
+    if (lse != nullptr && (reinterpret_cast<uintptr_t>(lse) & 3u) != 0) return FA_ERR_MISALIGNED;
+    fa::FwdParams p;
+    Shape shape{4, 2};
+    const int rc = validate(q, k, v, mask, out, B, R, L, H, stride_b, stride_h, stride_l, &p, scale,
+                            &shape, causal, lse);
+    if (rc != FA_OK) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (causal)
+        e = dispatch<fa::kCausal>(H, shape, p, s);
+    else if (mask != nullptr)
+        e = dispatch<fa::kAdditive>(H, shape, p, s);
+    else
+        e = dispatch<fa::kPlain>(H, shape, p, s);
+    return static_cast<int>(e);
+}
+
 int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,
            int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h, int64_t stride_l,
            float scale, void* stream) {
-    fa::FwdParams p;
-    Shape shape{4, 2};
-    const int rc = validate(q, k, v, mask, out, B, R, L, H, stride_b, stride_h, stride_l, &p, scale, &shape);
-    if (rc != FA_OK) return rc;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const hipError_t e = mask != nullptr ? dispatch<true>(H, shape, p, s) : dispatch<false>(H, shape, p, s);
-    return static_cast<int>(e);
+    return fa_fwd_ex(q, k, v, mask, out, nullptr, B, R, L, H, stride_b, stride_h, stride_l, scale, 0,
+                     stream);
 }
 
 int fa_fwd_timed(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,

@@ -46,6 +46,7 @@ struct FwdParams {
     const _Float16* v;
     const _Float16* mask;  // additive [B, L, L] or nullptr
     _Float16* o;
+    float* lse;            // optional [B, R, L] natural-log row sums of exp(scores), or nullptr
     int64_t stride_b;      // elements between batches
     int64_t stride_h;      // elements between heads
     int64_t stride_l;      // elements between sequence positions
@@ -57,6 +58,11 @@ struct FwdParams {
 };
 
 constexpr int kNumXcd = 8;
+
+// Kernel variants of the non-ping-pong kernel.
+constexpr int kPlain = 0;    // no mask: software-pipelined loop
+constexpr int kAdditive = 1; // additive [B, L, L] mask
+constexpr int kCausal = 2;   // key index <= query index, key tiles above the diagonal skipped
 
 template <int H>
 struct Geometry {
@@ -314,21 +320,31 @@ __device__ __forceinline__ void softmax_check(WaveState<H, NQB>& st, const float
     for (int nb = 0; nb < NQB; ++nb) st.l[nb] += ts[nb];
 }
 
-// Processes 32 keys (one sub-tile) for the wave's 64 queries, one stage after the other.  Used for
-// the ragged last tile and for the additive-mask variant.
+// Processes 32 keys (one sub-tile) for the wave's queries, one stage after the other.  Used for
+// the ragged last tile and for the additive-mask and causal variants.
 //   ks/vs : LDS tile base for the current buffer
 //   nvalid: number of valid keys in this sub-tile (only read when MASKED)
-template <int H, int NQB, bool MASKED, bool HAS_MASK>
+//   qrow  : sequence position of this lane's query in block 0 (block nb adds 32 nb); causal only
+template <int H, int NQB, bool MASKED, int MODE>
 __device__ __forceinline__ void process_subtile(WaveState<H, NQB>& st, const _Float16* ks,
                                                 const _Float16* vs, int sub, int nvalid,
                                                 float c, int lane,
                                                 const _Float16* const (&mask_row)[NQB],
-                                                int key_base, int L) {
+                                                int key_base, int L, int qrow = 0) {
     const int g = lane >> 5;
     floatx16 s[NQB];
     qk_mfma<H, NQB>(s, st.q, k_operand_ptr<H>(ks, sub, lane));
 
-    if constexpr (HAS_MASK) {
+    if constexpr (MODE == kCausal) {
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = key_base + 8 * (r >> 2) + 4 * g + (r & 3);
+                if (key > qrow + 32 * nb) s[nb][r] = -__builtin_inff();
+            }
+    }
+    if constexpr (MODE == kAdditive) {
 #pragma unroll
         for (int nb = 0; nb < NQB; ++nb) {
             const _Float16* mrow = mask_row[nb];
@@ -468,9 +484,11 @@ __device__ __forceinline__ void pipeline_stage(WaveState<H, NQB>& st, floatx16 (
 }
 
 // O = O^T / l in f32, one rounding to fp16, 8-byte stores of four consecutive head-dim elements.
+// With lse given (one float per query row of this (batch, head)), also writes
+// log(sum_j exp(score_j)) = m * scale + log(l), the quantity a backward pass needs.
 template <int H, int NQB>
 __device__ __forceinline__ void store_output(WaveState<H, NQB>& st, _Float16* obase, int64_t stride_l,
-                                             int q0, int L, int lane) {
+                                             int q0, int L, int lane, float* lse = nullptr, float c = 0.f) {
     using G = Geometry<H>;
     const int g = lane >> 5;
     const int ln = lane & 31;
@@ -480,6 +498,8 @@ __device__ __forceinline__ void store_output(WaveState<H, NQB>& st, _Float16* ob
         // A row whose every key carried a -inf mask has l = 0: emit zeros rather than NaN.
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
         const int row = q0 + nb * 32 + ln;
+        if (lse != nullptr && g == 0 && row < L)
+            lse[row] = lt > 0.f ? (st.m[nb] * c + __builtin_log2f(lt)) * 0.6931471805599453f : -__builtin_inff();
         if (row < L) {
             _Float16* orow = obase + (int64_t)row * stride_l;
 #pragma unroll
@@ -501,7 +521,7 @@ __device__ __forceinline__ void store_output(WaveState<H, NQB>& st, _Float16* ob
 
 // Template parameters: head_dim H, NW wave64s per workgroup, BK keys per LDS tile, NQB blocks of 32
 // query rows per wave, WPE waves per SIMD the register budget is sized for.
-template <int H, int NW, int BK, int NQB, int WPE, bool HAS_MASK>
+template <int H, int NW, int BK, int NQB, int WPE, int MODE>
 __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel(const FwdParams p) {
     using G = Geometry<H>;
     constexpr int QW = 32 * NQB;            // query rows per wave
@@ -572,34 +592,44 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel(const FwdParams p) {
     const int64_t sl = p.stride_l;
     TileLoader<H, NW, BK> loader;
 
-    if constexpr (HAS_MASK) {
-        // Additive-mask variant: plain double-buffered loop, one sub-tile after the other.
+    if constexpr (MODE != kPlain) {
+        // Additive-mask and causal variants: plain double-buffered loop, one sub-tile after the
+        // other.  Causal: the workgroup stops at the tile that holds its last query, and a wave
+        // skips the sub-tiles that lie entirely above its own last query.
         const _Float16* mask_row[NQB];
-        const _Float16* mb = p.mask + (int64_t)b * L * L;
 #pragma unroll
         for (int nb = 0; nb < NQB; ++nb) {
             const int row = q0 + nb * 32 + ln;
-            mask_row[nb] = row < L ? mb + (int64_t)row * L : nullptr;
+            mask_row[nb] = nullptr;
+            if constexpr (MODE == kAdditive)
+                if (row < L) mask_row[nb] = p.mask + (int64_t)b * L * L + (int64_t)row * L;
         }
+        int nt = ntiles;
+        if constexpr (MODE == kCausal) {
+            const int wg_last = min(qt * BQ + BQ, L) - 1;
+            nt = wg_last / BK + 1;
+        }
+        const int wave_last = q0 + QW - 1;
 
         loader.load_k(kbase, sl, 0, L, tid);
         loader.load_v(vbase, sl, 0, L, tid);
         loader.store_k(ks_base, tid);
         loader.store_v(vs_base, tid);
         __syncthreads();
-        for (int t = 0; t < ntiles; ++t) {
+        for (int t = 0; t < nt; ++t) {
             const int buf = t & 1;
-            const bool has_next = t + 1 < ntiles;
+            const bool has_next = t + 1 < nt;
             if (has_next) {
                 loader.load_k(kbase, sl, (t + 1) * BK, L, tid);
                 loader.load_v(vbase, sl, (t + 1) * BK, L, tid);
             }
 #pragma unroll
             for (int sub = 0; sub < NSUB; ++sub) {
-                const int nvalid = L - t * BK - sub * 32;
-                if (nvalid > 0)
-                    process_subtile<H, NQB, true, true>(st, ks_base + buf * KTILE, vs_base + buf * VTILE,
-                                                        sub, nvalid, c, lane, mask_row, t * BK + sub * 32, L);
+                const int key_base = t * BK + sub * 32;
+                const int nvalid = L - key_base;
+                if (nvalid > 0 && (MODE != kCausal || key_base <= wave_last))
+                    process_subtile<H, NQB, true, MODE>(st, ks_base + buf * KTILE, vs_base + buf * VTILE,
+                                                        sub, nvalid, c, lane, mask_row, key_base, L, q0 + ln);
             }
             if (has_next) {
                 loader.store_k(ks_base + (buf ^ 1) * KTILE, tid);
@@ -668,13 +698,14 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel(const FwdParams p) {
             for (int sub = 0; sub < NSUB; ++sub) {
                 const int nvalid = L - key0 - sub * 32;
                 if (nvalid > 0)
-                    process_subtile<H, NQB, true, false>(st, ks_base + buf * KTILE, vs_base + buf * VTILE,
-                                                         sub, nvalid, c, lane, no_mask, key0 + sub * 32, L);
+                    process_subtile<H, NQB, true, kPlain>(st, ks_base + buf * KTILE, vs_base + buf * VTILE,
+                                                          sub, nvalid, c, lane, no_mask, key0 + sub * 32, L);
             }
         }
     }
 
-    store_output<H, NQB>(st, obase, p.stride_l, q0, L, lane);
+    store_output<H, NQB>(st, obase, p.stride_l, q0, L, lane,
+                         p.lse != nullptr ? p.lse + ((int64_t)b * p.R + h) * L : nullptr, c);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -929,7 +960,8 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
     }
     if (grp == 0) phase_barrier();
 
-    store_output<H, NQB>(st, obase, sl, q0, L, lane);
+    store_output<H, NQB>(st, obase, sl, q0, L, lane,
+                         p.lse != nullptr ? p.lse + ((int64_t)b * p.R + h) * L : nullptr, c);
 }
 
 }  // namespace fa

@@ -32,6 +32,9 @@ extern "C" {
 #define FA_ERR_BAD_STRIDE (-4)
 #define FA_ERR_MISALIGNED (-5)
 #define FA_ERR_TOO_LARGE (-6)
+#define FA_ERR_BAD_FLAGS (-7)
+
+#define FA_FLAG_CAUSAL 1
 
 /*
  * out = softmax(q k^T * scale [+ mask]) v for every (batch, head), non-causal.
@@ -53,6 +56,23 @@ int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* 
            int64_t B, int64_t R, int64_t L, int64_t H,
            int64_t stride_b, int64_t stride_h, int64_t stride_l,
            float scale, void* stream);
+
+/*
+ * fa_fwd with two extensions the reference lists as not done yet (reference README.md:135-142,
+ * "backward pass", and its GPT/LLaMA use case, README.md:8):
+ *   flags & FA_FLAG_CAUSAL : query i attends to keys j <= i only; key tiles above the diagonal
+ *                            are skipped.  Not combinable with `mask`.
+ *   lse (nullable)         : float32 [B, R, L] in device memory, receives
+ *                            log(sum_j exp(score_ij)) per query row (-inf for a row whose keys
+ *                            are all masked): what a backward pass needs to recompute the
+ *                            probabilities.
+ * Everything else as fa_fwd, which is fa_fwd_ex with lse = NULL and flags = 0.  There is no
+ * counterpart in the reference (its kernel is non-causal and keeps no row statistics).
+ */
+int fa_fwd_ex(const void* q, const void* k, const void* v, const void* mask, void* out, void* lse,
+              int64_t B, int64_t R, int64_t L, int64_t H,
+              int64_t stride_b, int64_t stride_h, int64_t stride_l,
+              float scale, int flags, void* stream);
 
 /*
  * 1 if fa_fwd accepts this head_dim, else 0.  Counterpart of the compile-time

@@ -5,4 +5,5 @@ __graft_entry__.py and the cpu_baseline leg of bench.py may import it, and only 
 (or as the timed CPU baseline), never as the thing that computes a result handed to a user.
 The product path (fused_attention_amd, module fused_attn) never falls back to it.
 """
-from .naive_attention import attention, attention_per_head, attention_f64  # noqa: F401
+from .naive_attention import (attention, attention_f64, attention_lse, attention_per_head,  # noqa: F401
+                              causal_mask)

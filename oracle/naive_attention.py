@@ -54,6 +54,30 @@ def attention(queries, keys, values, head_dim, mask=None):
     return output.transpose(1, 2).contiguous().view(batch_size, sequence_len, num_features)
 
 
+def attention_lse(queries, keys, head_dim, mask=None):
+    """log(sum_j exp(score_ij)) of the scaled (and masked) scores, float32 [B, R, L].
+
+    The row statistic a backward pass needs; the reference's kernel does not produce it
+    (reference README.md:138-139 lists the backward pass as not done).  Pinned in
+    tests/test_oracle.py by closed forms: zero queries give log(L), and exp(score - lse) are the
+    softmax weights that reproduce `attention`.
+    """
+    batch_size, sequence_len, num_features = queries.shape
+    num_heads = num_features // head_dim
+    q = queries.to(torch.float32).view(batch_size, sequence_len, num_heads, head_dim).transpose(1, 2)
+    k = keys.to(torch.float32).view(batch_size, sequence_len, num_heads, head_dim).transpose(1, 2)
+    scores = (q @ k.mT) / (head_dim ** 0.5)
+    if mask is not None:
+        scores = scores + mask.to(torch.float32).view(batch_size, 1, sequence_len, sequence_len)
+    return torch.logsumexp(scores, dim=-1)
+
+
+def causal_mask(batch_size, sequence_len):
+    """Additive [B, L, L] mask of a causal model: 0 where key <= query, -inf above the diagonal."""
+    m = torch.full((sequence_len, sequence_len), float("-inf")).triu(1)
+    return m.expand(batch_size, sequence_len, sequence_len).contiguous()
+
+
 def attention_per_head(queries, keys, values, head_dim, heads=None):
     """Same arithmetic as `attention`, one (batch, head) at a time.
 

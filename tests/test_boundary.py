@@ -51,7 +51,10 @@ def test_status_codes_for_rejected_arguments():
     assert status(k_ptr=ok_ptr + 2) == -5
     assert status(L=2 ** 31) == -6
     assert status(B=2 ** 20, R=2 ** 20) == -6
-    for code in (-1, -2, -3, -4, -5, -6):
+    lib = capi.load_library()
+    assert lib.fa_fwd_ex(ok_ptr, ok_ptr, ok_ptr, None, ok_ptr, None, B, R, L, H, L * R * H, H, R * H, 0.125, 2, None) == -7
+    assert lib.fa_fwd_ex(ok_ptr, ok_ptr, ok_ptr, ok_ptr, ok_ptr, None, B, R, L, H, L * R * H, H, R * H, 0.125, 1, None) == -7
+    for code in (-1, -2, -3, -4, -5, -6, -7):
         assert "fa_fwd" in capi.strerror(code)
     assert capi.strerror(0) == "success"
 

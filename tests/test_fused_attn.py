@@ -14,7 +14,7 @@ import pytest
 import torch
 
 from fused_attention_amd import capi, workloads
-from oracle import attention, attention_per_head
+from oracle import attention, attention_lse, attention_per_head, causal_mask
 
 pytestmark = pytest.mark.gpu
 
@@ -230,6 +230,53 @@ def test_fully_masked_rows_give_zeros_not_nan(gpu):
     want = attention(q, k, v, H)
     keep = [i for i in range(L) if i not in (5, 77)]
     assert (out[0, keep] - want[0, keep]).abs().max().item() <= TOL
+
+
+# ---- causal flag and row log-sum-exp (extensions of the C ABI) -------------------------------------
+
+@pytest.mark.parametrize("B,R,L,H", [(1, 2, 64, 64), (2, 3, 200, 32), (1, 2, 777, 64), (2, 2, 300, 128),
+                                     (1, 12, 1024, 64), (1, 2, 33, 16)])
+def test_causal_matches_the_masked_oracle(gpu, B, R, L, H):
+    q, k, v = (_rand((B, L, R * H), 3700 + L + i) for i in range(3))
+    want = attention(q, k, v, H, mask=causal_mask(B, L))
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, causal=True)
+    assert _max_err(got, want) <= TOL
+    # the first row sees one key only: it returns V[0] exactly (after fp16 rounding of an fp16 value)
+    assert torch.equal(got[:, 0].cpu(), v[:, 0])
+
+
+@pytest.mark.parametrize("name,causal", [("c1", False), ("c2", False), ("c5a", False), ("c5a", True), ("c1", True)])
+def test_row_logsumexp(gpu, name, causal):
+    w = workloads.WORKLOADS[name]
+    q, k, v = workloads.make_inputs(w)
+    if w.B * w.R > 16:
+        q, k, v = (t[:1, :, : 4 * w.H].contiguous() for t in (q, k, v))
+    B, L, F = q.shape
+    mask = causal_mask(B, L) if causal else None
+    want_lse = attention_lse(q, k, w.H, mask=mask)
+    want_out = attention(q, k, v, w.H, mask=mask)
+    out, lse = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), w.H, causal=causal, return_lse=True)
+    assert lse.shape == (B, F // w.H, L) and lse.dtype == torch.float32
+    assert _max_err(out, want_out) <= TOL
+    # lse is an f32 quantity of magnitude up to ~40 on the stress inputs: compare relatively
+    assert ((lse.cpu() - want_lse).abs() / (1 + want_lse.abs())).max().item() <= 1e-3
+
+
+def test_lse_of_the_pingpong_kernel(gpu):
+    # enough workgroups to select the eight-wave kernel; zero queries give lse = log(L) exactly
+    B, R, L, H = 4, 16, 2048, 64
+    k, v = _rand((B, L, R * H), 3800), _rand((B, L, R * H), 3801)
+    out, lse = capi.forward(torch.zeros_like(k).to(gpu), k.to(gpu), v.to(gpu), H, return_lse=True)
+    assert (lse.cpu() - math.log(L)).abs().max().item() <= 1e-4
+    want = v.double().mean(dim=1, keepdim=True).float().expand(B, L, R * H)
+    assert _max_err(out, want) <= 1e-3
+
+
+def test_causal_with_mask_is_rejected(gpu):
+    x = torch.zeros(1, 64, 64, dtype=torch.float16, device=gpu)
+    m = torch.zeros(1, 64, 64, dtype=torch.float16, device=gpu)
+    with pytest.raises(capi.FusedAttnError):
+        capi.forward(x, x, x, 64, mask=m, causal=True)
 
 
 # ---- argument rejection that needs device tensors ---------------------------------------------------

@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 import torch
 
-from oracle import attention, attention_f64, attention_per_head
+from oracle import attention, attention_f64, attention_lse, attention_per_head, causal_mask
 
 ORACLE_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle")
 
@@ -166,3 +166,30 @@ def test_additive_mask_removes_keys():
     short = attention(*(t[:, :keep].contiguous() for t in (q, k, v)), H)
     torch.testing.assert_close(masked[:, :keep], short, rtol=0, atol=2e-6)
     np.testing.assert_allclose(masked.double().numpy(), _run_c(q, k, v, H, mask=mask), rtol=0, atol=2e-6)
+
+
+def test_lse_closed_forms():
+    B, R, L, H = 2, 2, 37, 32
+    q, k, v = (_rand((B, L, R * H), 110 + i) for i in range(3))
+    # zero queries: every score is 0, so lse = log(L)
+    lse0 = attention_lse(torch.zeros_like(q), k, H)
+    torch.testing.assert_close(lse0, torch.full((B, R, L), math.log(L)), rtol=0, atol=1e-6)
+    # exp(score - lse) are the softmax weights: they reproduce the attention output
+    lse = attention_lse(q, k, H)
+    qh = q.float().view(B, L, R, H).transpose(1, 2)
+    kh = k.float().view(B, L, R, H).transpose(1, 2)
+    vh = v.float().view(B, L, R, H).transpose(1, 2)
+    w = torch.exp((qh @ kh.mT) / math.sqrt(H) - lse.unsqueeze(-1))
+    torch.testing.assert_close(w.sum(-1), torch.ones(B, R, L), rtol=0, atol=1e-5)
+    out = (w @ vh).transpose(1, 2).reshape(B, L, R * H)
+    torch.testing.assert_close(out, attention(q, k, v, H), rtol=0, atol=1e-5)
+
+
+def test_causal_mask_means_prefix_attention():
+    # row i of the causal result equals the last row of the unmasked problem cut to i + 1 tokens
+    B, R, L, H = 1, 2, 21, 16
+    q, k, v = (_rand((B, L, R * H), 120 + i) for i in range(3))
+    causal = attention(q, k, v, H, mask=causal_mask(B, L))
+    for i in (0, 1, 7, L - 1):
+        prefix = attention(*(t[:, :i + 1].contiguous() for t in (q, k, v)), H)
+        torch.testing.assert_close(causal[:, i], prefix[:, i], rtol=0, atol=2e-6)
