@@ -23,23 +23,44 @@ struct Shape {
     int rows() const { return waves * 32 * nqb; }
 };
 
-// Three shapes, picked by how many workgroups the problem gives the 256 compute units:
-//   {8, 2}  eight 64-row waves share one K/V stream between 512 queries (head_dim <= 64, two
-//           waves per SIMD), run by the ping-pong kernel: best once every compute unit still gets
-//           two such workgroups; the additive-mask variant uses the plain eight-wave kernel;
-//   {4, 2}  four 64-row waves, 256 queries per workgroup;
+// Three shapes, picked by how the problem's workgroups fill the 256 compute units:
+//   {8, n}  eight waves of 64 (head_dim <= 64) or 32 (head_dim 128) query rows share one K/V
+//           stream, run by the ping-pong kernel; one such workgroup is resident per compute unit;
+//   {4, 2}  four 64-row waves, 256 queries per workgroup, two resident per compute unit;
 //   {4, 1}  four 32-row waves, 128 queries per workgroup, three (head_dim <= 64) or two
-//           (head_dim 128) waves per SIMD: more, smaller workgroups for short sequences.
-// head_dim 128 with 64-row waves needs the whole register file of a SIMD for one wave.
-Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask) {
+//           (head_dim 128) resident per compute unit: more, smaller workgroups for small problems.
+// head_dim 128 with 64-row waves needs the whole register file of a SIMD for one wave, and the
+// masked variants (additive mask, causal) exist only with four waves.
+int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
-    // the additive-mask variant at head_dim 128 only exists with 32-row waves (register budget)
-    if (H > 64 && has_mask) return {4, 1};
-    const int64_t wgs512 = B * R * ((L + 511) / 512);
-    const int64_t wgs256 = B * R * ((L + 255) / 256);
-    if (H > 64) return wgs256 >= 2 * kNumCu ? Shape{8, 1} : Shape{4, 1};
-    if (wgs512 >= 2 * kNumCu) return {8, 2};
-    return wgs256 >= 2 * kNumCu ? Shape{4, 2} : Shape{4, 1};
+// How well a shape uses the chip, in 1/1024: the share of the (rounds x slots) grid of resident
+// workgroup slots that the problem's workgroups occupy, times the share of each workgroup's query
+// rows that exist (the last workgroup of a sequence may be mostly empty).
+int64_t usage(int64_t heads, int64_t L, int64_t rows, int64_t slots) {
+    const int64_t per_head = ceil_div(L, rows);
+    const int64_t wgs = heads * per_head;
+    return wgs * L * 1024 / (ceil_div(wgs, slots) * slots * per_head * rows);
+}
+
+Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool masked) {
+    const int64_t heads = B * R;
+    if (masked) {
+        if (H > 64) return {4, 1};
+        return heads * ceil_div(L, 256) >= 2 * kNumCu ? Shape{4, 2} : Shape{4, 1};
+    }
+    // The ping-pong kernel is the fastest per compute unit, so it is taken whenever its
+    // workgroups fill the chip well enough.  Thresholds measured on MI355X: a lone round may be
+    // emptier than the tail of several, because idle units leave the busy ones more of the
+    // power budget.
+    const int64_t rows8 = H > 64 ? 256 : 512;
+    const int64_t wgs8 = heads * ceil_div(L, rows8);
+    const int64_t usage8 = usage(heads, L, rows8, kNumCu);
+    const bool pingpong = wgs8 >= 2 * kNumCu ? usage8 >= 614 : usage8 >= (wgs8 <= kNumCu ? 614 : 717);
+    if (H > 64) return pingpong ? Shape{8, 1} : Shape{4, 1};
+    if (pingpong) return {8, 2};
+    // everything resident at once: the smallest workgroups give the most parallelism
+    if (heads * ceil_div(L, 128) <= 3 * kNumCu) return {4, 1};
+    return usage(heads, L, 256, 2 * kNumCu) > usage(heads, L, 128, 3 * kNumCu) ? Shape{4, 2} : Shape{4, 1};
 }
 
 // Dynamic LDS above 64 KiB has to be opted into per kernel function and per device: done on the

@@ -272,6 +272,54 @@ def test_lse_of_the_pingpong_kernel(gpu):
     assert _max_err(out, want) <= 1e-3
 
 
+# ---- every launch shape, plain and masked -------------------------------------------------------------
+
+def _check_pairs(got, q, k, v, H, pairs, mask=None):
+    """Compares the listed (batch, head) slices of a full-tensor result against the oracle."""
+    for b, h in pairs:
+        sl = slice(h * H, (h + 1) * H)
+        want = attention(q[b:b + 1, :, sl], k[b:b + 1, :, sl], v[b:b + 1, :, sl], H,
+                         mask=None if mask is None else mask[b:b + 1])
+        assert _max_err(got[b:b + 1, :, sl], want) <= TOL, (b, h)
+
+
+@pytest.mark.parametrize("B,R,L,H", [
+    (1, 20, 4096, 64),      # eight-wave workgroups filling part of one round of the chip
+    (1, 40, 4096, 64),      # a poorly filled second round: four-wave workgroups instead
+    (1, 500, 256, 64),      # short sequences, 64-row waves
+    (4, 16, 2112, 64),      # many workgroups, ragged last key tile and last query tile
+    (1, 20, 2048, 128),     # head_dim 128, eight-wave workgroups in a part-filled round
+    (1, 40, 2048, 128),     # head_dim 128, four-wave workgroups
+    (2, 160, 1088, 128),    # head_dim 128, many workgroups, ragged tiles
+])
+def test_launch_shapes_plain(gpu, B, R, L, H):
+    q, k, v = (_rand((B, L, R * H), 3900 + L + i) for i in range(3))
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H)
+    assert torch.isfinite(got.float()).all()
+    _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R // 2), (B - 1, R - 1)])
+
+
+@pytest.mark.parametrize("B,R,L,H", [(4, 16, 4096, 64), (8, 64, 512, 64), (2, 64, 1024, 128), (3, 100, 300, 32)])
+def test_causal_on_large_grids(gpu, B, R, L, H):
+    q, k, v = (_rand((B, L, R * H), 3950 + L + i) for i in range(3))
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, causal=True)
+    assert torch.isfinite(got.float()).all()
+    _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R // 2), (B - 1, R - 1)], mask=causal_mask(B, L))
+    assert torch.equal(got[:, 0].cpu(), v[:, 0])
+
+
+@pytest.mark.parametrize("B,R,L,H", [(8, 64, 512, 64), (4, 40, 700, 128), (16, 40, 384, 16)])
+def test_additive_mask_on_large_grids(gpu, B, R, L, H):
+    q, k, v = (_rand((B, L, R * H), 3970 + L + i) for i in range(3))
+    g = torch.Generator().manual_seed(3975)
+    mask = torch.where(torch.rand(B, L, L, generator=g) < 0.3, float("-inf"), 0.0)
+    mask = (mask + torch.randn(B, L, L, generator=g) * 0.5).to(torch.float16)
+    mask[:, :, 0] = 0
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, mask=mask.to(gpu))
+    assert torch.isfinite(got.float()).all()
+    _check_pairs(got, q, k, v, H, [(0, 0), (B // 2, R // 2), (B - 1, R - 1)], mask=mask.float())
+
+
 def test_causal_with_mask_is_rejected(gpu):
     x = torch.zeros(1, 64, 64, dtype=torch.float16, device=gpu)
     m = torch.zeros(1, 64, 64, dtype=torch.float16, device=gpu)
