@@ -147,6 +147,8 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     if (mask != nullptr && (reinterpret_cast<uintptr_t>(mask) & 1u) != 0) return FA_ERR_MISALIGNED;
     constexpr int64_t kMaxInt = 0x7fffffff;
     if (L > kMaxInt - 4096 || B > kMaxInt || R > kMaxInt) return FA_ERR_TOO_LARGE;
+    // the tile loaders keep 32-bit byte offsets inside a 64-key tile
+    if (stride_l > ((int64_t)1 << 24)) return FA_ERR_TOO_LARGE;
     *shape = pick_shape(B, R, L, H, mask != nullptr || causal);
     const int64_t bq = shape->rows();
     const int64_t n_qtiles = (L + bq - 1) / bq;

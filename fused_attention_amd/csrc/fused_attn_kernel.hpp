@@ -120,19 +120,35 @@ struct TileLoader {
     static constexpr bool EXACT = NCHUNK % NT == 0;
     u32x4 kreg[NP];
     u32x4 vreg[NP];
+    uint32_t goff[NP];   // byte offset of this thread's chunk i from the first key of a tile
 
-    // Rows at or beyond L are read from row L - 1 instead of being predicated off (a predicated
-    // load into a zeroed register makes every load wait for the one before it).  Such keys are
-    // masked to -inf before the softmax, and a probability of exactly zero times a finite V row
-    // contributes nothing.
-    static __device__ __forceinline__ void load(u32x4 (&reg)[NP], const _Float16* base, int64_t stride_l,
-                                                int key0, int L, int tid) {
-        if (key0 >= L) return;
+    __device__ __forceinline__ void init(int64_t stride_l, int tid) {
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
             const int idx = EXACT ? tid + i * NT : min(tid + i * NT, NCHUNK - 1);
-            const int key = min(key0 + idx / CPR, L - 1);
-            reg[i] = *reinterpret_cast<const u32x4*>(base + (int64_t)key * stride_l + (idx % CPR) * 8);
+            goff[i] = (uint32_t)(((int64_t)(idx / CPR) * stride_l + (idx % CPR) * 8) * 2);
+        }
+    }
+
+    // A full tile is fetched with one uniform base address plus the per-thread byte offsets (no
+    // vector address arithmetic inside the key loop).  In the ragged last tile, rows at or beyond
+    // L are read from row L - 1 instead of being predicated off (a predicated load into a zeroed
+    // register makes every load wait for the one before it).  Such keys are masked to -inf before
+    // the softmax, and a probability of exactly zero times a finite V row contributes nothing.
+    __device__ __forceinline__ void load(u32x4 (&reg)[NP], const _Float16* base, int64_t stride_l,
+                                         int key0, int L, int tid) const {
+        if (key0 >= L) return;
+        if (key0 + BK <= L) {
+            const char* tile = reinterpret_cast<const char*>(base + (int64_t)key0 * stride_l);
+#pragma unroll
+            for (int i = 0; i < NP; ++i) reg[i] = *reinterpret_cast<const u32x4*>(tile + goff[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < NP; ++i) {
+                const int idx = EXACT ? tid + i * NT : min(tid + i * NT, NCHUNK - 1);
+                const int key = min(key0 + idx / CPR, L - 1);
+                reg[i] = *reinterpret_cast<const u32x4*>(base + (int64_t)key * stride_l + (idx % CPR) * 8);
+            }
         }
     }
     template <int STR>
@@ -591,6 +607,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel(const FwdParams p) {
     const float c = p.scale_log2e;
     const int64_t sl = p.stride_l;
     TileLoader<H, NW, BK> loader;
+    loader.init(sl, tid);
 
     if constexpr (MODE != kPlain) {
         // Additive-mask and causal variants: plain double-buffered loop, one sub-tile after the

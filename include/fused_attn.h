@@ -50,7 +50,8 @@ extern "C" {
  *   - `mask` (nullable) is an additive fp16 [B, L, L] tensor shared by all heads and is
  *     applied to every key, not only to the first chunk.  Rows whose keys are all -inf
  *     produce zeros.
- * B, R, L >= 1.  L*stride_l, R*stride_h and B*stride_b must stay below 2^62 elements.
+ * B, R, L >= 1.  L*stride_l, R*stride_h and B*stride_b must stay below 2^62 elements and
+ * stride_l must not exceed 2^24 elements (FA_ERR_TOO_LARGE otherwise).
  */
 int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* out,
            int64_t B, int64_t R, int64_t L, int64_t H,
