@@ -30,7 +30,7 @@ struct Shape {
 //   {4, 1}  four 32-row waves, 128 queries per workgroup, three (head_dim <= 64) or two
 //           (head_dim 128) resident per compute unit: more, smaller workgroups for small problems.
 // head_dim 128 with 64-row waves needs the whole register file of a SIMD for one wave, and the
-// masked variants (additive mask, causal) exist only with four waves.
+// additive-mask variant exists only with four waves.
 int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // How well a shape uses the chip, in 1/1024: the share of the (rounds x slots) grid of resident
@@ -42,17 +42,18 @@ int64_t usage(int64_t heads, int64_t L, int64_t rows, int64_t slots) {
     return wgs * L * 1024 / (ceil_div(wgs, slots) * slots * per_head * rows);
 }
 
-Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool masked) {
+Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask, bool causal) {
     const int64_t heads = B * R;
-    if (masked) {
+    // the additive-mask variant exists only with four waves
+    if (has_mask) {
         if (H > 64) return {4, 1};
         return heads * ceil_div(L, 256) >= 2 * kNumCu ? Shape{4, 2} : Shape{4, 1};
     }
     // The ping-pong kernel is the fastest per compute unit, so it is taken whenever its
     // workgroups fill the chip well enough.  Thresholds measured on MI355X: a lone round may be
     // emptier than the tail of several, because idle units leave the busy ones more of the
-    // power budget.
-    const int64_t rows8 = H > 64 ? 256 : 512;
+    // power budget.  A causal ping-pong workgroup takes two query tiles (see the kernel).
+    const int64_t rows8 = (H > 64 ? 256 : 512) * (causal ? 2 : 1);
     const int64_t wgs8 = heads * ceil_div(L, rows8);
     const int64_t usage8 = usage(heads, L, rows8, kNumCu);
     const bool pingpong = wgs8 >= 2 * kNumCu ? usage8 >= 614 : usage8 >= (wgs8 <= kNumCu ? 614 : 717);
@@ -92,10 +93,10 @@ hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
-template <int H, int NW, int NQB, int WPE>
+template <int H, int NW, int NQB, int WPE, bool CAUSAL>
 hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
     constexpr int lds = fa::lds_bytes_pingpong<H, NQB>();
-    auto kernel = fa::fwd_kernel_pingpong<H, NW, NQB, WPE>;
+    auto kernel = fa::fwd_kernel_pingpong<H, NW, NQB, WPE, CAUSAL>;
     if constexpr (lds > 64 * 1024) {
         const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), lds);
         if (e != hipSuccess) return e;
@@ -107,19 +108,20 @@ hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
 
 template <int H, int MODE>
 hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) {
-    if constexpr (MODE != fa::kPlain) {
-        // masked variants: four waves, 64-row waves where the registers allow it
-        if constexpr (H > 64)
-            return launch<H, 4, 1, 2, MODE>(p, stream);
-        else
-            return sh.nqb == 2 ? launch<H, 4, 2, 2, MODE>(p, stream) : launch<H, 4, 1, 3, MODE>(p, stream);
-    } else if constexpr (H > 64) {
-        if (sh.waves == 8) return launch_pingpong<H, 8, 1, 2>(p, stream);
-        return sh.nqb == 2 ? launch<H, 4, 2, 1, MODE>(p, stream) : launch<H, 4, 1, 2, MODE>(p, stream);
-    } else {
-        if (sh.waves == 8) return launch_pingpong<H, 8, 2, 2>(p, stream);
-        return sh.nqb == 2 ? launch<H, 4, 2, 2, MODE>(p, stream) : launch<H, 4, 1, 3, MODE>(p, stream);
+    if constexpr (MODE != fa::kAdditive) {
+        // plain and causal: the ping-pong kernel for the eight-wave shapes
+        if (sh.waves == 8) {
+            if constexpr (H > 64)
+                return launch_pingpong<H, 8, 1, 2, MODE == fa::kCausal>(p, stream);
+            else
+                return launch_pingpong<H, 8, 2, 2, MODE == fa::kCausal>(p, stream);
+        }
     }
+    // four waves: 64-row waves where the registers allow it
+    if constexpr (H > 64)
+        return launch<H, 4, 1, 2, MODE>(p, stream);
+    else
+        return sh.nqb == 2 ? launch<H, 4, 2, 2, MODE>(p, stream) : launch<H, 4, 1, 3, MODE>(p, stream);
 }
 
 template <int MODE>
@@ -149,9 +151,10 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     if (L > kMaxInt - 4096 || B > kMaxInt || R > kMaxInt) return FA_ERR_TOO_LARGE;
     // the tile loaders keep 32-bit byte offsets inside a 64-key tile
     if (stride_l > ((int64_t)1 << 24)) return FA_ERR_TOO_LARGE;
-    *shape = pick_shape(B, R, L, H, mask != nullptr || causal);
+    *shape = pick_shape(B, R, L, H, mask != nullptr, causal);
     const int64_t bq = shape->rows();
-    const int64_t n_qtiles = (L + bq - 1) / bq;
+    int64_t n_qtiles = (L + bq - 1) / bq;
+    if (causal && shape->waves == 8) n_qtiles = (n_qtiles + 1) / 2;   // pairs of query tiles
     const int64_t total = B * R * n_qtiles;
     if (total > kMaxInt - 8 || B * R > kMaxInt) return FA_ERR_TOO_LARGE;
     constexpr int64_t kMaxElems = (int64_t)1 << 62;

@@ -51,7 +51,8 @@ struct FwdParams {
     int64_t stride_h;      // elements between heads
     int64_t stride_l;      // elements between sequence positions
     int B, R, L;
-    int n_qtiles;          // ceil(L / queries per workgroup)
+    int n_qtiles;          // workgroups per (batch, head): ceil(L / queries per workgroup), or half of
+                           // that (rounded up) when a causal workgroup takes a pair of query tiles
     int total_wgs;         // B * R * n_qtiles
     int wgs_per_xcd;       // ceil(total_wgs / 8)
     float scale_log2e;     // scale * log2(e)
@@ -564,7 +565,8 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel(const FwdParams p) {
     const int logical = (wg % kNumXcd) * p.wgs_per_xcd + wg / kNumXcd;
     if (logical >= p.total_wgs) return;
     const int bh = logical / p.n_qtiles;
-    const int qt = logical % p.n_qtiles;
+    // causal: longest-running query tiles of a head first
+    const int qt = MODE == kCausal ? p.n_qtiles - 1 - logical % p.n_qtiles : logical % p.n_qtiles;
     const int b = bh / p.R;
     const int h = bh % p.R;
     const int L = p.L;
@@ -782,8 +784,9 @@ struct GroupLoader {
     // Rows at or beyond L are read from row L - 1 instead (no predicated loads, so no load ever
     // waits for another): their scores are masked to -inf, or belong to sub-tiles that are never
     // consumed, and a probability of exactly zero times a finite V row contributes nothing.
-    __device__ __forceinline__ void load(const _Float16* src, int64_t stride_l, int key0, int L) {
-        if (key0 >= L) return;
+    // Tiles starting at or beyond `limit` are not fetched at all (limit <= L).
+    __device__ __forceinline__ void load(const _Float16* src, int64_t stride_l, int key0, int limit, int L) {
+        if (key0 >= limit) return;
         if (key0 + 64 <= L && EXACT) {
             const _Float16* tile = src + (int64_t)key0 * stride_l;
 #pragma unroll
@@ -803,7 +806,7 @@ struct GroupLoader {
     }
 };
 
-template <int H, int NW, int NQB, int WPE>
+template <int H, int NW, int NQB, int WPE, bool CAUSAL>
 __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdParams p) {
     using G = Geometry<H>;
     constexpr int BK = 64;
@@ -831,8 +834,12 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
     const int wg = blockIdx.x;
     const int logical = (wg % kNumXcd) * p.wgs_per_xcd + wg / kNumXcd;
     if (logical >= p.total_wgs) return;
+    // Causal: query tile t of a head costs t + 1 key blocks, so a workgroup takes two tiles, t and
+    // n_qtiles - 1 - t, one after the other: every workgroup of the grid then does the same amount
+    // of work, whatever order the hardware hands them out in.  p.n_qtiles counts these pairs.
+    const int tiles_per_head = (p.L + BQ - 1) / BQ;
     const int bh = logical / p.n_qtiles;
-    const int qt = logical % p.n_qtiles;
+    const int slot = logical % p.n_qtiles;
     const int b = bh / p.R;
     const int h = bh % p.R;
     const int L = p.L;
@@ -842,13 +849,17 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
     const _Float16* kbase = p.k + head_off;
     const _Float16* vbase = p.v + head_off;
     _Float16* obase = p.o + head_off;
-    const int q0 = qt * BQ + wave * QW;
     const int64_t sl = p.stride_l;
 
     if constexpr (G::HV != H) {
         for (int i = tid; i < 3 * VTILE; i += NW * 64) vs_base[i] = (_Float16)0.f;
         __syncthreads();
     }
+
+    for (int pass = 0; pass < (CAUSAL ? 2 : 1); ++pass) {
+    const int qt = CAUSAL ? (pass == 0 ? tiles_per_head - 1 - slot : slot) : slot;
+    if (CAUSAL && pass == 1 && 2 * slot == tiles_per_head - 1) break;   // middle tile of an odd count
+    const int q0 = qt * BQ + wave * QW;
 
     WaveState<H, NQB> st;
 #pragma unroll
@@ -871,8 +882,13 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
     }
 
     const float c = p.scale_log2e;
-    const int nsub = (L + 31) >> 5;
-    const int last_valid = L - (nsub - 1) * 32;     // valid keys in the last sub-tile (1..32)
+    // causal: the workgroup stops at the sub-tile that holds its last query, and each wave at the
+    // sub-tile that holds its own last query (nact); after that a wave only keeps up its share of
+    // the K/V streaming and the barriers
+    const int Lk = CAUSAL ? min(qt * BQ + BQ, L) : L;
+    const int nsub = (Lk + 31) >> 5;
+    const int last_valid = Lk - (nsub - 1) * 32;    // valid keys in the last sub-tile (1..32)
+    const int nact = CAUSAL ? min(nsub, (q0 + QW) >> 5) : nsub;
 
     // Group 0 streams K, group 1 streams V.
     GroupLoader<H, GT> gl;
@@ -882,11 +898,11 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
     const int ring_tile = grp == 0 ? KTILE : VTILE;
 
     // prologue: tiles 0 and 1 into the ring, tile 2 into registers
-    gl.load(gsrc, sl, 0, L);
+    gl.load(gsrc, sl, 0, Lk, L);
     gl.store(ring);
-    gl.load(gsrc, sl, BK, L);
+    gl.load(gsrc, sl, BK, Lk, L);
     gl.store(ring + ring_tile);
-    gl.load(gsrc, sl, 2 * BK, L);
+    gl.load(gsrc, sl, 2 * BK, Lk, L);
     __syncthreads();
 
     floatx16 s[NQB];
@@ -895,7 +911,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
     qk_mfma<H, NQB>(s, st.q, k_operand_ptr<H>(ks_base, 0, lane));
     if (grp == 1) phase_barrier();                  // the second group runs one phase behind
 
-    for (int j = 0; j < nsub; ++j) {
+    for (int j = 0; j < nact; ++j) {
         const int T = j >> 1;
         const int jn = j + 1;
         // ---- vector phase -------------------------------------------------------------------
@@ -935,6 +951,17 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
                 }
             }
         }
+        if constexpr (CAUSAL) {
+            if (j * 32 + 31 > q0) {     // the sub-tile reaches above the diagonal for some of the wave's queries
+#pragma unroll
+                for (int nb = 0; nb < NQB; ++nb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int key = j * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+                        if (key > q0 + 32 * nb + ln) s[nb][r] = -__builtin_inff();
+                    }
+            }
+        }
         exp_pack_sum<NQB>(s, c, st.mc, pk, ts);
         softmax_check<H, NQB>(st, s, c, pk, ts);
         phase_barrier();
@@ -972,13 +999,23 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
         }
         // the global loads of the tile three ahead go last: they cost this wave a few issue slots
         // while its matrix instructions are already queued
-        if ((j & 1) == 0) gl.load(gsrc, sl, (T + 3) * BK, L);
+        if ((j & 1) == 0) gl.load(gsrc, sl, (T + 3) * BK, Lk, L);
         phase_barrier();
+    }
+    if constexpr (CAUSAL) {
+        for (int j = nact; j < nsub; ++j) {
+            const int T = j >> 1;
+            if ((j & 1) == 0) gl.store(ring + ((T + 2) % 3) * ring_tile);
+            phase_barrier();
+            if ((j & 1) == 0) gl.load(gsrc, sl, (T + 3) * BK, Lk, L);
+            phase_barrier();
+        }
     }
     if (grp == 0) phase_barrier();
 
     store_output<H, NQB>(st, obase, sl, q0, L, lane,
                          p.lse != nullptr ? p.lse + ((int64_t)b * p.R + h) * L : nullptr, c);
+    }   // pass
 }
 
 }  // namespace fa

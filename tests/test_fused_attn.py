@@ -299,13 +299,25 @@ def test_launch_shapes_plain(gpu, B, R, L, H):
     _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R // 2), (B - 1, R - 1)])
 
 
-@pytest.mark.parametrize("B,R,L,H", [(4, 16, 4096, 64), (8, 64, 512, 64), (2, 64, 1024, 128), (3, 100, 300, 32)])
+@pytest.mark.parametrize("B,R,L,H", [
+    (4, 16, 4096, 64),      # eight-wave workgroups, each taking a pair of query tiles (8 tiles per head)
+    (2, 64, 1300, 64),      # ... with an odd number of tiles (the middle one runs alone) and a ragged end
+    (2, 64, 1024, 128),     # head_dim 128, four tiles of 256 queries
+    (4, 64, 1250, 128),     # head_dim 128, five tiles, ragged end
+    (8, 64, 512, 64), (3, 100, 300, 32),     # four-wave workgroups
+])
 def test_causal_on_large_grids(gpu, B, R, L, H):
     q, k, v = (_rand((B, L, R * H), 3950 + L + i) for i in range(3))
-    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, causal=True)
+    got, lse = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, causal=True, return_lse=True)
     assert torch.isfinite(got.float()).all()
-    _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R // 2), (B - 1, R - 1)], mask=causal_mask(B, L))
+    mask = causal_mask(B, L)
+    pairs = [(0, 0), (B - 1, R // 2), (B - 1, R - 1)]
+    _check_pairs(got, q, k, v, H, pairs, mask=mask)
     assert torch.equal(got[:, 0].cpu(), v[:, 0])
+    for b, h in pairs:
+        sl = slice(h * H, (h + 1) * H)
+        want = attention_lse(q[b:b + 1, :, sl], k[b:b + 1, :, sl], H, mask=mask[b:b + 1])[0, 0]
+        assert ((lse[b, h].cpu() - want).abs() / (1 + want.abs())).max().item() <= 1e-3
 
 
 @pytest.mark.parametrize("B,R,L,H", [(8, 64, 512, 64), (4, 40, 700, 128), (16, 40, 384, 16)])
