@@ -347,8 +347,33 @@ __device__ __forceinline__ void process_subtile(WaveState<H, NQB>& st, const _Fl
                                                 const _Float16* vs, int sub, int nvalid,
                                                 float c, int lane,
                                                 const _Float16* const (&mask_row)[NQB],
-                                                int key_base, int L, int qrow = 0) {
+                                                int key_base, int L, int qrow = 0, bool mask_vec = false) {
     const int g = lane >> 5;
+    // Additive mask: this lane's 16 keys of the sub-tile are four runs of four consecutive keys.
+    // The mask values are fetched before the first product so that their latency hides behind it:
+    // as 8-byte loads when every run is 8-byte aligned and entirely inside the row (L % 4 == 0 and
+    // an aligned mask pointer, which `mask_vec` says), as single fp16 loads otherwise.
+    half4 mk[NQB][4];
+    if constexpr (MODE == kAdditive) {
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb) {
+            const _Float16* mrow = mask_row[nb];
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int key = key_base + 8 * r4 + 4 * g;
+                mk[nb][r4] = half4{(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+                if (mrow != nullptr) {
+                    if (mask_vec) {
+                        if (key < L) mk[nb][r4] = *reinterpret_cast<const half4*>(mrow + key);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (key + j < L) mk[nb][r4][j] = mrow[key + j];
+                    }
+                }
+            }
+        }
+    }
     floatx16 s[NQB];
     qk_mfma<H, NQB>(s, st.q, k_operand_ptr<H>(ks, sub, lane));
 
@@ -362,24 +387,13 @@ __device__ __forceinline__ void process_subtile(WaveState<H, NQB>& st, const _Fl
             }
     }
     if constexpr (MODE == kAdditive) {
+        // The mask is added to the scaled score; S holds raw scores, so the mask is brought to raw
+        // units: s * scale + mask = scale * (s + mask / scale).
+        const float inv_scale = 1.4426950408889634f / c;
 #pragma unroll
-        for (int nb = 0; nb < NQB; ++nb) {
-            const _Float16* mrow = mask_row[nb];
-            if (mrow != nullptr) {
+        for (int nb = 0; nb < NQB; ++nb)
 #pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    const int key = key_base + 8 * r4 + 4 * g;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if (key + j < L) {
-                            // The mask is added to the scaled score; S holds raw scores, so the
-                            // mask is brought to raw units: s*scale + mask = scale*(s + mask/scale).
-                            s[nb][4 * r4 + j] += (float)mrow[key + j] * (1.4426950408889634f / c);
-                        }
-                    }
-                }
-            }
-        }
+            for (int r = 0; r < 16; ++r) s[nb][r] += (float)mk[nb][r >> 2][r & 3] * inv_scale;
     }
     if constexpr (MASKED) {
 #pragma unroll
@@ -629,6 +643,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel(const FwdParams p) {
             nt = wg_last / BK + 1;
         }
         const int wave_last = q0 + QW - 1;
+        const bool mask_vec = MODE == kAdditive && (L & 3) == 0 && (reinterpret_cast<uintptr_t>(p.mask) & 7) == 0;
 
         loader.load_k(kbase, sl, 0, L, tid);
         loader.load_v(vbase, sl, 0, L, tid);
@@ -648,7 +663,8 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel(const FwdParams p) {
                 const int nvalid = L - key_base;
                 if (nvalid > 0 && (MODE != kCausal || key_base <= wave_last))
                     process_subtile<H, NQB, true, MODE>(st, ks_base + buf * KTILE, vs_base + buf * VTILE,
-                                                        sub, nvalid, c, lane, mask_row, key_base, L, q0 + ln);
+                                                        sub, nvalid, c, lane, mask_row, key_base, L, q0 + ln,
+                                                        mask_vec);
             }
             if (has_next) {
                 loader.store_k(ks_base + (buf ^ 1) * KTILE, tid);

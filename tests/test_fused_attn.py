@@ -203,8 +203,11 @@ def test_heads_and_batches_are_independent_bitwise(gpu):
 
 # ---- additive mask ---------------------------------------------------------------------------------
 
-@pytest.mark.parametrize("L,H", [(64, 64), (200, 32), (300, 128)])
-def test_additive_mask_on_every_key_tile(gpu, L, H):
+@pytest.mark.parametrize("L,H,offset", [(64, 64, 0), (200, 32, 0), (300, 128, 0), (203, 64, 0), (97, 16, 0),
+                                        (200, 64, 1)])
+def test_additive_mask_on_every_key_tile(gpu, L, H, offset):
+    # L % 4 != 0 or a mask that starts `offset` elements into its allocation (2-byte aligned only)
+    # take the element-wise mask loads instead of the 8-byte ones
     import fused_attn
 
     B, R = 2, 2
@@ -214,7 +217,11 @@ def test_additive_mask_on_every_key_tile(gpu, L, H):
     mask = (mask + torch.randn(B, L, L, generator=g) * 0.5).to(torch.float16)
     mask[:, :, 0] = 0                                   # keep at least one key per row
     want = attention(q, k, v, H, mask=mask)
-    got = fused_attn.attention_forward(H, 32, q.to(gpu), k.to(gpu), v.to(gpu), mask.to(gpu))
+    flat = torch.empty(B * L * L + offset, dtype=torch.float16, device=gpu)
+    dev_mask = flat[offset:].view(B, L, L)
+    dev_mask.copy_(mask)
+    assert dev_mask.is_contiguous() and dev_mask.data_ptr() % 8 == (2 * offset) % 8
+    got = fused_attn.attention_forward(H, 32, q.to(gpu), k.to(gpu), v.to(gpu), dev_mask)
     assert _max_err(got, want) <= TOL
 
 
