@@ -1,0 +1,223 @@
+// Instruction-issue probes for gfx950, run as `fa_test issue-probe`: how matrix (MFMA) and vector
+// (VALU) instructions of one or two waves on the same SIMD overlap.  The attention kernels are
+// scheduled around these numbers.  A 512-thread workgroup places waves w and w + 4 on the same
+// SIMD; all figures are shader clocks (s_memtime) per instruction or per group of instructions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+
+namespace probe {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+#define PROBE_OK(expr)                                                                        \
+    do {                                                                                      \
+        hipError_t e_ = (expr);                                                               \
+        if (e_ != hipSuccess) {                                                               \
+            std::fprintf(stderr, "%s failed: %s\n", #expr, hipGetErrorString(e_));            \
+            return 2;                                                                         \
+        }                                                                                     \
+    } while (0)
+
+#define P_FMA(d, s) asm volatile("v_fma_f32 %0, %1, %2, %3" : "=v"(d) : "v"(s), "v"(a), "v"(b))
+#define P_EXP(d) asm volatile("v_exp_f32 %0, %0" : "+v"(d))
+#define P_CVT(d, x, y) asm volatile("v_cvt_pkrtz_f16_f32 %0, %1, %2" : "=v"(d) : "v"(x), "v"(y))
+#define P_DOT(acc, x) asm volatile("v_dot2c_f32_f16 %0, %1, %2" : "+v"(acc) : "v"(0x3c003c00u), "v"(x))
+#define P_MFMA(c) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(x), "v"(y))
+
+// Probe 1: waves 0-3 issue MFMAs only, waves 4-7 (same SIMDs) one kind of vector instruction only.
+// mode bit 0: matrix waves run, bit 1: vector waves run.  VK: 0 fma, 1 exp, 2 cvt_pkrtz, 3 dot2c.
+template <int VK>
+__global__ __launch_bounds__(512) void split_kernel(long long* out, const h8* data, int iters, int mode,
+                                                    float a, float b) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    long long t0 = 0, t1 = 0;
+    float sink = 0.f;
+    if (wave < 4) {
+        if (!(mode & 1)) return;
+        const h8 x = data[threadIdx.x], y = data[threadIdx.x + 512];
+        f16v c[4];
+        for (int n = 0; n < 4; n++)
+            for (int r = 0; r < 16; r++) c[n][r] = 0.f;
+        t0 = clock64();
+        for (int it = 0; it < iters; it++) {
+#pragma unroll
+            for (int j = 0; j < 16; j++) P_MFMA(c[j & 3]);
+        }
+        t1 = clock64();
+        for (int n = 0; n < 4; n++)
+            for (int r = 0; r < 16; r++) sink += c[n][r];
+    } else {
+        if (!(mode & 2)) return;
+        float v[8];
+        for (int i = 0; i < 8; i++) v[i] = a * (lane + i);
+        unsigned pk[4] = {0, 0, 0, 0};
+        t0 = clock64();
+        for (int it = 0; it < iters; it++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                if (VK == 0) asm volatile("v_fma_f32 %0, %1, %0, %2" : "+v"(v[i & 7]) : "v"(a), "v"(b));
+                if (VK == 1) P_EXP(v[i & 7]);
+                if (VK == 2) P_CVT(pk[i & 3], v[i & 7], v[(i + 1) & 7]);
+                if (VK == 3) P_DOT(v[i & 7], pk[i & 3]);
+            }
+        }
+        t1 = clock64();
+        for (int i = 0; i < 8; i++) sink += v[i];
+        for (int i = 0; i < 4; i++) sink += (float)pk[i];
+    }
+    if (lane == 0) out[wave] = t1 - t0;
+    if (sink == 1.2345f) out[8] = 1;
+}
+
+// Probe 2: every wave loops over {1 MFMA, N independent vector instructions}.
+template <int N, int VK>
+__global__ __launch_bounds__(512) void mixed_kernel(long long* out, const h8* data, int iters, float a, float b) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const h8 x = data[threadIdx.x], y = data[threadIdx.x + 512];
+    f16v c[4];
+    for (int n = 0; n < 4; n++)
+        for (int r = 0; r < 16; r++) c[n][r] = 0.f;
+    float v[8];
+    for (int i = 0; i < 8; i++) v[i] = a * (lane + i);
+    const long long t0 = clock64();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            P_MFMA(c[j & 3]);
+#pragma unroll
+            for (int i = 0; i < N; i++) {
+                if (VK == 0) asm volatile("v_fma_f32 %0, %1, %0, %2" : "+v"(v[(j * N + i) & 7]) : "v"(a), "v"(b));
+                else P_EXP(v[(j * N + i) & 7]);
+            }
+        }
+    }
+    const long long t1 = clock64();
+    float sink = 0.f;
+    for (int n = 0; n < 4; n++)
+        for (int r = 0; r < 16; r++) sink += c[n][r];
+    for (int i = 0; i < 8; i++) sink += v[i];
+    if (lane == 0) out[wave] = t1 - t0;
+    if (sink == 1.2345f) out[8] = 1;
+}
+
+// Probe 3: the softmax chunk of the attention kernels (2 fma, 2 exp, 1 pack, 1 dot2 for one fp16
+// pair of probabilities) with or without one MFMA per chunk.
+// PAT 0: chunk + MFMA, 1: chunk without the dot2 + MFMA, 2: chunks only, 3: MFMAs only.
+template <int PAT>
+__global__ __launch_bounds__(512) void chunk_kernel(long long* out, const h8* data, int iters, float a, float b) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const h8 x = data[threadIdx.x], y = data[threadIdx.x + 512];
+    f16v c[4];
+    for (int n = 0; n < 4; n++)
+        for (int r = 0; r < 16; r++) c[n][r] = 0.f;
+    float s[16];
+    for (int i = 0; i < 16; i++) s[i] = -0.01f * (lane + i);
+    unsigned pk[8] = {};
+    float acc = 0.f, e0 = 0.f, e1 = 0.f;
+    const long long t0 = clock64();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (PAT != 3) {
+                float n0, n1;
+                P_FMA(n0, s[2 * i]);
+                P_FMA(n1, s[2 * i + 1]);
+                P_EXP(n0);
+                P_EXP(n1);
+                P_CVT(pk[i], e0, e1);      // the pair exponentiated one chunk earlier
+                if (PAT != 1) P_DOT(acc, pk[i]);
+                e0 = n0;
+                e1 = n1;
+            }
+            if (PAT != 2) P_MFMA(c[i & 3]);
+        }
+    }
+    const long long t1 = clock64();
+    float sink = acc + e0 + e1;
+    for (int n = 0; n < 4; n++)
+        for (int r = 0; r < 16; r++) sink += c[n][r];
+    for (int i = 0; i < 8; i++) sink += (float)pk[i];
+    if (lane == 0) out[wave] = t1 - t0;
+    if (sink == 1.2345f) out[8] = 1;
+}
+
+template <int VK>
+int run_split(const char* name, long long* d, const h8* data) {
+    const int iters = 2000;
+    long long h[8];
+    double res[4][2] = {};
+    for (int mode = 1; mode <= 3; mode++) {
+        PROBE_OK(hipMemset(d, 0, 128));
+        for (int rep = 0; rep < 2; rep++)
+            hipLaunchKernelGGL(split_kernel<VK>, dim3(1), dim3(512), 0, 0, d, data, iters, mode, 0.999f, 0.001f);
+        PROBE_OK(hipDeviceSynchronize());
+        PROBE_OK(hipMemcpy(h, d, sizeof(h), hipMemcpyDeviceToHost));
+        res[mode][0] = (double)h[0] / (iters * 16.0);
+        res[mode][1] = (double)h[4] / (iters * 16.0);
+    }
+    std::printf("  %-10s alone: %5.1f clk/mfma, %5.1f clk/%s | together: %5.1f clk/mfma, %5.1f clk/%s\n", name,
+                res[1][0], res[2][1], name, res[3][0], res[3][1], name);
+    return 0;
+}
+
+template <int N, int VK>
+int run_mixed(long long* d, const h8* data) {
+    const int iters = 2000;
+    long long h[8];
+    for (int rep = 0; rep < 2; rep++)
+        hipLaunchKernelGGL((mixed_kernel<N, VK>), dim3(1), dim3(256), 0, 0, d, data, iters, 0.999f, 0.001f);
+    PROBE_OK(hipDeviceSynchronize());
+    PROBE_OK(hipMemcpy(h, d, sizeof(h), hipMemcpyDeviceToHost));
+    std::printf("  {1 mfma + %d %s}: %5.1f clk\n", N, VK ? "exp" : "fma", (double)h[0] / (iters * 8.0));
+    return 0;
+}
+
+template <int PAT>
+int run_chunk(const char* name, long long* d, const h8* data) {
+    const int iters = 2000;
+    for (int threads : {256, 512}) {
+        long long h[8];
+        for (int rep = 0; rep < 2; rep++)
+            hipLaunchKernelGGL(chunk_kernel<PAT>, dim3(1), dim3(threads), 0, 0, d, data, iters, 0.999f, 0.001f);
+        PROBE_OK(hipDeviceSynchronize());
+        PROBE_OK(hipMemcpy(h, d, sizeof(h), hipMemcpyDeviceToHost));
+        std::printf("  %-28s %d wave(s) per SIMD: oldest wave %5.1f, youngest wave %5.1f clk per chunk\n", name,
+                    threads / 256, (double)h[0] / (iters * 8.0), (double)h[threads / 64 - 1] / (iters * 8.0));
+    }
+    return 0;
+}
+
+inline int issue_probe() {
+    long long* d;
+    h8* data;
+    PROBE_OK(hipMalloc(&d, 4096));
+    PROBE_OK(hipMalloc(&data, 16 * 1024));
+    PROBE_OK(hipMemset(data, 0, 16 * 1024));
+    std::printf("issue-probe 1: a matrix wave and a vector wave on the same SIMD (v_mfma_f32_32x32x16_f16)\n");
+    run_split<0>("fma", d, data);
+    run_split<1>("exp", d, data);
+    run_split<2>("cvt_pkrtz", d, data);
+    run_split<3>("dot2c", d, data);
+    std::printf("issue-probe 2: one wave per SIMD issuing both kinds\n");
+    run_mixed<0, 0>(d, data);
+    run_mixed<2, 0>(d, data);
+    run_mixed<4, 0>(d, data);
+    run_mixed<6, 0>(d, data);
+    run_mixed<8, 0>(d, data);
+    run_mixed<2, 1>(d, data);
+    run_mixed<4, 1>(d, data);
+    std::printf("issue-probe 3: softmax chunk {2 fma, 2 exp, 1 pack, 1 dot2} with one MFMA per chunk\n");
+    run_chunk<0>("chunk + mfma", d, data);
+    run_chunk<1>("chunk without dot2 + mfma", d, data);
+    run_chunk<2>("chunks only", d, data);
+    run_chunk<3>("mfma only", d, data);
+    (void)hipFree(d);
+    (void)hipFree(data);
+    return 0;
+}
+
+}  // namespace probe
