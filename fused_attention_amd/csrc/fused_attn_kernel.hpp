@@ -744,13 +744,20 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel(const FwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Ping-pong variant: eight waves per workgroup, two per SIMD.  On this hardware a wave does not
-// overlap its own vector work with its own matrix instructions, so the overlap has to come from
-// the two waves that share a SIMD.  The waves form two groups (0-3 and 4-7, one wave of each per
-// SIMD) that alternate between a vector phase (exponentials of sub-tile j) and a matrix phase
-// (PV of sub-tile j, QK^T of sub-tile j + 1), the second group one phase behind the first, with a
-// workgroup barrier between phases: while one group keeps the matrix cores busy the other does
-// the softmax on the vector ALUs of the same SIMDs.
+// Ping-pong variant: eight waves per workgroup, two per SIMD.  A SIMD picks between its waves
+// oldest first, so two free-running waves do not share it evenly: the older one runs at nearly
+// its single-wave speed, the younger one fills the gaps, and they drift apart (measured by
+// `fa_test issue-probe`).  Here the two waves of a SIMD are kept in step instead.  The waves form
+// two groups (0-3 and 4-7, one wave of each per SIMD) that alternate between a vector phase
+// (exponentials of sub-tile j) and a matrix phase (PV of sub-tile j, QK^T of sub-tile j + 1), the
+// second group one phase behind the first, with a workgroup barrier between phases: while one
+// group keeps the matrix cores busy the other does the softmax on the vector ALUs of the same SIMDs.
+//
+// Causal (CAUSAL = true): a wave stops computing at the sub-tile that holds its last query and then
+// only keeps up its share of the K/V streaming and of the barriers; scores above the diagonal are
+// set to -inf in the (at most three) sub-tiles that straddle it.  Query tile t of a head costs
+// t + 1 key blocks, so a workgroup takes the tiles t and n - 1 - t one after the other and all
+// workgroups of the grid do the same amount of work.
 //
 // K and V stream through three-slot LDS rings.  Group 0 loads K, group 1 loads V, each during its
 // own vector phases: at its first vector phase of tile T a group writes tile T + 2 (fetched into
