@@ -35,6 +35,7 @@ typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
@@ -196,6 +197,57 @@ __device__ __forceinline__ void exp_pack_sum(const floatx16 (&s)[NQB], float c, 
     }
 }
 
+// Same exponentials without the sums: returns the bitwise OR of all packed fp16 pairs of the
+// sub-tile.  A non-negative fp16 value is below 2.0 exactly when bit 14 is clear (inf and NaN have
+// it set), so the OR tells whether any probability of the sub-tile reached 2.0.  The reference the
+// exponentials are taken against carries a bias of kBias (log2 units) on top of the running row
+// maximum: probabilities normally stay below 2^-kBias, and the fast path tolerates a reference
+// that lags the true maximum by up to kBias + 1.  The factor 2^-kBias cancels between O and l; the
+// smallest probabilities lose kBias bits of fp16 sub-normal range, far below the rounding of O.
+constexpr float kBias = 6.0f;
+constexpr uint32_t kTripBits = 0x40004000u;
+template <int NQB>
+__device__ __forceinline__ uint32_t exp_pack_or(const floatx16 (&s)[NQB], float c, const float (&mc)[NQB],
+                                                uint32_t (&pk)[NQB][8]) {
+    uint32_t orv = 0u;
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) {
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nb][r], c, mc[nb]));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nb][r + 1], c, mc[nb]));
+            const uint32_t pp = pack_rtz(p0, p1);
+            pk[nb][r >> 1] = pp;
+            orv |= pp;
+        }
+    }
+    return orv;
+}
+__device__ __forceinline__ bool trips(uint32_t orv) { return (orv & kTripBits) != 0u; }
+
+// A operand that makes v_mfma_f32_16x16x32_f16 add up the packed P^T registers of one k-step per
+// query.  In that instruction lane l holds A[l % 16][8 (l / 16) + i] and B[8 (l / 16) + i][l % 16],
+// and D[m][n] lands in lane n + 16 (m / 4), register m % 4.  Read as its B operand, the P^T registers
+// of lane l hold eight keys of query l % 32, i.e. column n = l % 16 carries query n in k-blocks 0
+// and 2 and query n + 16 in k-blocks 1 and 3.  With row 0 of A selecting k-blocks 0 and 2 and row 4
+// selecting k-blocks 1 and 3, register 0 of lane q (q < 32) receives the sum over the 16 keys of
+// query q: the lane that owns the query.  Lanes 32..63 receive zeros.
+__device__ __forceinline__ half8 row_sum_operand(int lane) {
+    const _Float16 v = (lane == 0 || lane == 32 || lane == 20 || lane == 52) ? (_Float16)1.0f : (_Float16)0.f;
+    const half8 a = {v, v, v, v, v, v, v, v};
+    return a;
+}
+template <int NQB>
+__device__ __forceinline__ void row_sum_mfma(floatx4 (&lacc)[NQB], half8 sel, const uint32_t (&pk)[NQB][8]) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb) {
+            const u32x4 w = {pk[nb][4 * t], pk[nb][4 * t + 1], pk[nb][4 * t + 2], pk[nb][4 * t + 3]};
+            lacc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(sel, __builtin_bit_cast(half8, w), lacc[nb], 0, 0, 0);
+        }
+}
+
 // O^T[.][nb] *= alpha, in place.  Written as one instruction per register with the register tied
 // as input and output, so that the rarely taken rescale does not make the compiler keep a second
 // copy of the accumulators (and copy them on the common path).  The leading wait covers the
@@ -224,6 +276,7 @@ struct WaveState {
     float m[NQB];   // reference row maximum of the raw (unscaled) scores, identical in lanes l and l^32
     float mc[NQB];  // -m * c, the additive term of the exponent; +inf while no reference exists yet
     float l[NQB];   // running sum of exp over the keys this lane has seen (half of each tile)
+    floatx4 lacc[NQB];  // ping-pong kernel: row sums accumulated by the matrix core, see row_sum_mfma
 };
 
 // LDS address of this lane's K row for sub-tile `sub` of a tile: A operand of S^T = K_sub * Q^T.
@@ -291,13 +344,12 @@ __device__ __forceinline__ void pv_mfma(floatx16 (&o)[Geometry<H>::DB][NQB], con
     }
 }
 
-// Slow path of the online softmax: bring the reference up to the true running maximum of the rows,
-// rescale O and l, and redo the exponentials of this sub-tile against the new reference.
+// Slow path of the online softmax, first part: bring the reference up to the true running maximum
+// of the rows and rescale O and l.  mcu receives the exponent term to redo this sub-tile with.
 template <int H, int NQB>
-__device__ __forceinline__ void softmax_fix(WaveState<H, NQB>& st, const floatx16 (&s)[NQB], float c,
-                                         uint32_t (&pk)[NQB][8], float (&ts)[NQB]) {
+__device__ __forceinline__ void softmax_rebase(WaveState<H, NQB>& st, const floatx16 (&s)[NQB], float c,
+                                               float (&mcu)[NQB], float bias = 0.f) {
     using G = Geometry<H>;
-    float mcu[NQB];
 #pragma unroll
     for (int nb = 0; nb < NQB; ++nb) {
         float mx = fmax2(s[nb][0], s[nb][1]);
@@ -312,11 +364,20 @@ __device__ __forceinline__ void softmax_fix(WaveState<H, NQB>& st, const floatx1
         const bool empty = m_new == -__builtin_inff();
         const float alpha = empty ? 1.f : __builtin_amdgcn_exp2f((m_old - m_new) * c);
         st.l[nb] *= alpha;
+        st.lacc[nb][0] *= alpha;
         scale_accumulators<G::DB, NQB>(st.o, nb, alpha);
         st.m[nb] = m_new;
-        st.mc[nb] = empty ? __builtin_inff() : -m_new * c;
-        mcu[nb] = empty ? 0.f : -m_new * c;
+        st.mc[nb] = empty ? __builtin_inff() : -m_new * c - bias;
+        mcu[nb] = empty ? 0.f : -m_new * c - bias;
     }
+}
+
+// ... second part: redo the exponentials of this sub-tile against the new reference.
+template <int H, int NQB>
+__device__ __forceinline__ void softmax_fix(WaveState<H, NQB>& st, const floatx16 (&s)[NQB], float c,
+                                         uint32_t (&pk)[NQB][8], float (&ts)[NQB]) {
+    float mcu[NQB];
+    softmax_rebase<H, NQB>(st, s, c, mcu);
     exp_pack_sum<NQB>(s, c, mcu, pk, ts);
 }
 
@@ -519,7 +580,8 @@ __device__ __forceinline__ void pipeline_stage(WaveState<H, NQB>& st, floatx16 (
 // log(sum_j exp(score_j)) = m * scale + log(l), the quantity a backward pass needs.
 template <int H, int NQB>
 __device__ __forceinline__ void store_output(WaveState<H, NQB>& st, _Float16* obase, int64_t stride_l,
-                                             int q0, int L, int lane, float* lse = nullptr, float c = 0.f) {
+                                             int q0, int L, int lane, float* lse = nullptr, float c = 0.f,
+                                             float l_bias = 0.f) {
     using G = Geometry<H>;
     const int g = lane >> 5;
     const int ln = lane & 31;
@@ -530,7 +592,7 @@ __device__ __forceinline__ void store_output(WaveState<H, NQB>& st, _Float16* ob
         const float inv = lt > 0.f ? 1.0f / lt : 0.f;
         const int row = q0 + nb * 32 + ln;
         if (lse != nullptr && g == 0 && row < L)
-            lse[row] = lt > 0.f ? (st.m[nb] * c + __builtin_log2f(lt)) * 0.6931471805599453f : -__builtin_inff();
+            lse[row] = lt > 0.f ? (st.m[nb] * c + __builtin_log2f(lt) + l_bias) * 0.6931471805599453f : -__builtin_inff();
         if (row < L) {
             _Float16* orow = obase + (int64_t)row * stride_l;
 #pragma unroll
@@ -898,6 +960,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
         st.m[nb] = -__builtin_inff();
         st.mc[nb] = __builtin_inff();
         st.l[nb] = 0.f;
+        st.lacc[nb] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int db = 0; db < G::DB; ++db)
 #pragma unroll
@@ -930,7 +993,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
 
     floatx16 s[NQB];
     uint32_t pk[NQB][8];
-    float ts[NQB];
+    const half8 sel = row_sum_operand(lane);
     qk_mfma<H, NQB>(s, st.q, k_operand_ptr<H>(ks_base, 0, lane));
     if (grp == 1) phase_barrier();                  // the second group runs one phase behind
 
@@ -985,8 +1048,13 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
                     }
             }
         }
-        exp_pack_sum<NQB>(s, c, st.mc, pk, ts);
-        softmax_check<H, NQB>(st, s, c, pk, ts);
+        // Exponentials against the reference maximum of the rows seen so far; the row sums are left
+        // to the matrix phase (row_sum_mfma), the overflow check works on the packed values.
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(trips(exp_pack_or<NQB>(s, c, st.mc, pk))) != 0, 0)) {
+            float mcu[NQB];
+            softmax_rebase<H, NQB>(st, s, c, mcu, kBias);
+            exp_pack_or<NQB>(s, c, mcu, pk);
+        }
         phase_barrier();
         // ---- matrix phase -------------------------------------------------------------------
 #pragma unroll
@@ -1020,6 +1088,7 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
                 }
             }
         }
+        row_sum_mfma<NQB>(st.lacc, sel, pk);
         // the global loads of the tile three ahead go last: they cost this wave a few issue slots
         // while its matrix instructions are already queued
         if ((j & 1) == 0) gl.load(gsrc, sl, (T + 3) * BK, Lk, L);
@@ -1036,8 +1105,10 @@ __global__ __launch_bounds__(NW * 64, WPE) void fwd_kernel_pingpong(const FwdPar
     }
     if (grp == 0) phase_barrier();
 
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) st.l[nb] = st.lacc[nb][0];
     store_output<H, NQB>(st, obase, sl, q0, L, lane,
-                         p.lse != nullptr ? p.lse + ((int64_t)b * p.R + h) * L : nullptr, c);
+                         p.lse != nullptr ? p.lse + ((int64_t)b * p.R + h) * L : nullptr, c, kBias);
     }   // pass
 }
 

@@ -306,6 +306,30 @@ def test_launch_shapes_plain(gpu, B, R, L, H):
     _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R // 2), (B - 1, R - 1)])
 
 
+@pytest.mark.parametrize("B,R,L,H", [(4, 16, 2048, 64), (2, 64, 1024, 128)])
+@pytest.mark.parametrize("kind", ["std3", "rising", "falling"])
+def test_eight_wave_kernel_on_adversarial_scores(gpu, B, R, L, H, kind):
+    # Grids large enough for the eight-wave kernel, with scores that stress its running reference
+    # maximum: |score| > 20 all over (std3), or a score that climbs (falls) by about 100 along the
+    # key axis, so that the reference is overtaken again and again (never after the first key).
+    q, k, v = (_rand((B, L, R * H), 4100 + L + i) for i in range(3))
+    if kind == "std3":
+        q, k = (q.float() * 3).half(), (k.float() * 3).half()
+    else:
+        g = torch.Generator().manual_seed(4107)
+        u = torch.randn(R * H, generator=g)
+        u = u / u.view(R, H).norm(dim=1).repeat_interleave(H)           # unit vector per head
+        ramp = torch.linspace(0, 1, L) if kind == "rising" else torch.linspace(1, 0, L)
+        q = (q.float() * 0.3 + 10.0 * u).half()
+        k = (k.float() * 0.3 + (10.0 * math.sqrt(H)) * ramp.view(1, L, 1) * u).half()
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H)
+    assert torch.isfinite(got.float()).all()
+    _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R // 2), (B - 1, R - 1)])
+    sl = slice(0, H)
+    scores = (q[0, :, sl].float() @ k[0, :, sl].float().T) / math.sqrt(H)
+    assert scores.abs().max() > 20
+
+
 @pytest.mark.parametrize("B,R,L,H", [
     (4, 16, 4096, 64),      # eight-wave workgroups, each taking a pair of query tiles (8 tiles per head)
     (2, 64, 1300, 64),      # ... with an odd number of tiles (the middle one runs alone) and a ragged end
