@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libfused_attn_gfx950.so")
 # every symbol include/fused_attn.h declares
 EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_query", "fa_strerror", "fa_fwd_timed")
 FLAG_CAUSAL = 1
+FLAG_BF16 = 2
 
 _lib = None
 
@@ -87,14 +88,21 @@ def _current_stream(q):
 
 def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None, causal=False,
             return_lse=False):
-    """Runs fa_fwd_ex on torch GPU tensors (fp16, contiguous) on torch's current stream.
+    """Runs fa_fwd_ex on torch GPU tensors (fp16 or bf16, contiguous) on torch's current stream.
 
     layout 'blf' takes [B, L, R*head_dim] tensors, 'bhld' takes [B, R, L, head_dim] tensors.
-    causal=True restricts query i to keys j <= i.  Returns `out` (allocated like q when not
+    causal=True restricts query i to keys j <= i.  q, k, v (and out, mask when given) must share
+    one dtype; bfloat16 tensors set FA_FLAG_BF16.  Returns `out` (allocated like q when not
     given), or (out, lse) with lse a float32 [B, R, L] tensor when return_lse is set.
     """
     import torch
 
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("q, k, v must be float16 or bfloat16, got %s" % q.dtype)
+    for name, t in (("k", k), ("v", v), ("out", out), ("mask", mask)):
+        if t is not None and t.dtype != q.dtype:
+            raise TypeError("%s must have the dtype of q (%s), got %s" % (name, q.dtype, t.dtype))
+    flags = (FLAG_CAUSAL if causal else 0) | (FLAG_BF16 if q.dtype == torch.bfloat16 else 0)
     B, R, L, sb, sh, sl = _layout(q, head_dim, layout)
     if out is None:
         out = torch.empty_like(q)
@@ -105,7 +113,7 @@ def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None, ca
         status = load_library().fa_fwd_ex(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr() if mask is not None else None,
             out.data_ptr(), lse.data_ptr() if lse is not None else None, B, R, L, head_dim, sb, sh, sl,
-            scale, FLAG_CAUSAL if causal else 0, _current_stream(q) or None)
+            scale, flags, _current_stream(q) or None)
     _check(status)
     return (out, lse) if return_lse else out
 

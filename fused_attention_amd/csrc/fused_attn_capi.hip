@@ -80,10 +80,11 @@ hipError_t allow_large_lds(const void* kernel, int bytes) {
     return e;
 }
 
-template <int H, int NW, int NQB, int WPE, int MODE>
+// BF selects the bf16 instantiation (namespace fa::bf16) of the same kernel source.
+template <int H, int NW, int NQB, int WPE, int MODE, bool BF>
 hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
     constexpr int lds = fa::lds_bytes<H, NW, kKeyTile>();
-    auto kernel = fa::fwd_kernel<H, NW, kKeyTile, NQB, WPE, MODE>;
+    auto kernel = BF ? fa::bf16::fwd_kernel<H, NW, kKeyTile, NQB, WPE, MODE> : fa::fwd_kernel<H, NW, kKeyTile, NQB, WPE, MODE>;
     if constexpr (lds > 64 * 1024) {
         const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), lds);
         if (e != hipSuccess) return e;
@@ -93,10 +94,10 @@ hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
-template <int H, int NW, int NQB, int WPE, bool CAUSAL>
+template <int H, int NW, int NQB, int WPE, bool CAUSAL, bool BF>
 hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
     constexpr int lds = fa::lds_bytes_pingpong<H, NQB>();
-    auto kernel = fa::fwd_kernel_pingpong<H, NW, NQB, WPE, CAUSAL>;
+    auto kernel = BF ? fa::bf16::fwd_kernel_pingpong<H, NW, NQB, WPE, CAUSAL> : fa::fwd_kernel_pingpong<H, NW, NQB, WPE, CAUSAL>;
     if constexpr (lds > 64 * 1024) {
         const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), lds);
         if (e != hipSuccess) return e;
@@ -106,33 +107,38 @@ hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
-template <int H, int MODE>
+template <int H, int MODE, bool BF>
 hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) {
     if constexpr (MODE != fa::kAdditive) {
         // plain and causal: the ping-pong kernel for the eight-wave shapes
         if (sh.waves == 8) {
             if constexpr (H > 64)
-                return launch_pingpong<H, 8, 1, 2, MODE == fa::kCausal>(p, stream);
+                return launch_pingpong<H, 8, 1, 2, MODE == fa::kCausal, BF>(p, stream);
             else
-                return launch_pingpong<H, 8, 2, 2, MODE == fa::kCausal>(p, stream);
+                return launch_pingpong<H, 8, 2, 2, MODE == fa::kCausal, BF>(p, stream);
         }
     }
     // four waves: 64-row waves where the registers allow it
     if constexpr (H > 64)
-        return launch<H, 4, 1, 2, MODE>(p, stream);
+        return launch<H, 4, 1, 2, MODE, BF>(p, stream);
     else
-        return sh.nqb == 2 ? launch<H, 4, 2, 2, MODE>(p, stream) : launch<H, 4, 1, 3, MODE>(p, stream);
+        return sh.nqb == 2 ? launch<H, 4, 2, 2, MODE, BF>(p, stream) : launch<H, 4, 1, 3, MODE, BF>(p, stream);
+}
+
+template <int MODE, bool BF>
+hipError_t dispatch_head_dim(int64_t H, Shape sh, const fa::FwdParams& p, hipStream_t stream) {
+    switch (H) {
+        case 16: return dispatch_shape<16, MODE, BF>(sh, p, stream);
+        case 32: return dispatch_shape<32, MODE, BF>(sh, p, stream);
+        case 64: return dispatch_shape<64, MODE, BF>(sh, p, stream);
+        case 128: return dispatch_shape<128, MODE, BF>(sh, p, stream);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 template <int MODE>
-hipError_t dispatch(int64_t H, Shape sh, const fa::FwdParams& p, hipStream_t stream) {
-    switch (H) {
-        case 16: return dispatch_shape<16, MODE>(sh, p, stream);
-        case 32: return dispatch_shape<32, MODE>(sh, p, stream);
-        case 64: return dispatch_shape<64, MODE>(sh, p, stream);
-        case 128: return dispatch_shape<128, MODE>(sh, p, stream);
-        default: return hipErrorInvalidValue;
-    }
+hipError_t dispatch(int64_t H, Shape sh, const fa::FwdParams& p, hipStream_t stream, bool bf16) {
+    return bf16 ? dispatch_head_dim<MODE, true>(H, sh, p, stream) : dispatch_head_dim<MODE, false>(H, sh, p, stream);
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
@@ -207,8 +213,9 @@ const char* fa_strerror(int status) {
 int fa_fwd_ex(const void* q, const void* k, const void* v, const void* mask, void* out, void* lse,
               int64_t B, int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h,
               int64_t stride_l, float scale, int flags, void* stream) {
-    if ((flags & ~FA_FLAG_CAUSAL) != 0) return FA_ERR_BAD_FLAGS;
+    if ((flags & ~(FA_FLAG_CAUSAL | FA_FLAG_BF16)) != 0) return FA_ERR_BAD_FLAGS;
     const bool causal = (flags & FA_FLAG_CAUSAL) != 0;
+    const bool bf16 = (flags & FA_FLAG_BF16) != 0;
     if (causal && mask != nullptr) return FA_ERR_BAD_FLAGS;
     if (lse != nullptr && (reinterpret_cast<uintptr_t>(lse) & 3u) != 0) return FA_ERR_MISALIGNED;
     fa::FwdParams p;
@@ -219,11 +226,11 @@ int fa_fwd_ex(const void* q, const void* k, const void* v, const void* mask, voi
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e;
     if (causal)
-        e = dispatch<fa::kCausal>(H, shape, p, s);
+        e = dispatch<fa::kCausal>(H, shape, p, s, bf16);
     else if (mask != nullptr)
-        e = dispatch<fa::kAdditive>(H, shape, p, s);
+        e = dispatch<fa::kAdditive>(H, shape, p, s, bf16);
     else
-        e = dispatch<fa::kPlain>(H, shape, p, s);
+        e = dispatch<fa::kPlain>(H, shape, p, s, bf16);
     return static_cast<int>(e);
 }
 

@@ -35,6 +35,7 @@ extern "C" {
 #define FA_ERR_BAD_FLAGS (-7)
 
 #define FA_FLAG_CAUSAL 1
+#define FA_FLAG_BF16 2
 
 /*
  * out = softmax(q k^T * scale [+ mask]) v for every (batch, head), non-causal.
@@ -63,6 +64,9 @@ int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* 
  * "backward pass", and its GPT/LLaMA use case, README.md:8):
  *   flags & FA_FLAG_CAUSAL : query i attends to keys j <= i only; key tiles above the diagonal
  *                            are skipped.  Not combinable with `mask`.
+ *   flags & FA_FLAG_BF16   : q, k, v, out (and mask) hold bfloat16 instead of fp16 (reference
+ *                            README.md:137 lists other input types as not done).  Same kernels,
+ *                            bf16 matrix instructions, probabilities rounded to bf16.
  *   lse (nullable)         : float32 [B, R, L] in device memory, receives
  *                            log(sum_j exp(score_ij)) per query row (-inf for a row whose keys
  *                            are all masked): what a backward pass needs to recompute the

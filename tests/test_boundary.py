@@ -53,7 +53,7 @@ def test_status_codes_for_rejected_arguments():
     assert status(B=2 ** 20, R=2 ** 20) == -6
     assert status(stride_l=2 ** 24 + 8, stride_b=2 ** 40) == -6   # row pitch beyond the loaders' 32-bit tile offsets
     lib = capi.load_library()
-    assert lib.fa_fwd_ex(ok_ptr, ok_ptr, ok_ptr, None, ok_ptr, None, B, R, L, H, L * R * H, H, R * H, 0.125, 2, None) == -7
+    assert lib.fa_fwd_ex(ok_ptr, ok_ptr, ok_ptr, None, ok_ptr, None, B, R, L, H, L * R * H, H, R * H, 0.125, 4, None) == -7
     assert lib.fa_fwd_ex(ok_ptr, ok_ptr, ok_ptr, ok_ptr, ok_ptr, None, B, R, L, H, L * R * H, H, R * H, 0.125, 1, None) == -7
     for code in (-1, -2, -3, -4, -5, -6, -7):
         assert "fa_fwd" in capi.strerror(code)

@@ -363,6 +363,51 @@ def test_additive_mask_on_large_grids(gpu, B, R, L, H):
     _check_pairs(got, q, k, v, H, [(0, 0), (B // 2, R // 2), (B - 1, R - 1)], mask=mask.float())
 
 
+# ---- bfloat16 inputs (FA_FLAG_BF16) ------------------------------------------------------------------
+
+BF16_TOL = 2e-2   # bf16 keeps 8 significant bits: the output rounding alone is 2^-9 * |o|
+
+
+@pytest.mark.parametrize("B,R,L,H,causal", [
+    (1, 2, 64, 64, False), (2, 3, 200, 32, False), (1, 2, 333, 16, True), (2, 2, 300, 128, False),
+    (4, 16, 2048, 64, False), (4, 16, 2048, 64, True),       # eight-wave kernel
+    (2, 64, 1024, 128, False), (2, 64, 1024, 128, True),
+    (2, 8, 1000, 64, False),
+])
+def test_bf16_inputs(gpu, B, R, L, H, causal):
+    q, k, v = (_rand((B, L, R * H), 4200 + L + i).to(torch.bfloat16) for i in range(3))
+    got, lse = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, causal=causal, return_lse=True)
+    assert got.dtype == torch.bfloat16 and torch.isfinite(got.float()).all()
+    mask = causal_mask(B, L) if causal else None
+    pairs = sorted({(0, 0), (B - 1, R // 2), (B - 1, R - 1)})
+    for b, h in pairs:
+        sl = slice(h * H, (h + 1) * H)
+        m = None if mask is None else mask[b:b + 1]
+        want = attention(q[b:b + 1, :, sl], k[b:b + 1, :, sl], v[b:b + 1, :, sl], H, mask=m)
+        assert _max_err(got[b:b + 1, :, sl], want) <= BF16_TOL, (b, h)
+        want_lse = attention_lse(q[b:b + 1, :, sl], k[b:b + 1, :, sl], H, mask=m)[0, 0]
+        assert ((lse[b, h].cpu() - want_lse).abs() / (1 + want_lse.abs())).max().item() <= 2e-3
+
+
+def test_bf16_additive_mask_and_closed_forms(gpu):
+    B, R, L, H = 2, 2, 200, 64
+    q, k, v = (_rand((B, L, R * H), 4300 + i).to(torch.bfloat16) for i in range(3))
+    g = torch.Generator().manual_seed(4310)
+    mask = torch.where(torch.rand(B, L, L, generator=g) < 0.3, float("-inf"), 0.0)
+    mask = (mask + torch.randn(B, L, L, generator=g) * 0.5).to(torch.bfloat16)
+    mask[:, :, 0] = 0
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, mask=mask.to(gpu))
+    assert _max_err(got, attention(q, k, v, H, mask=mask)) <= BF16_TOL
+    # constant V comes back exactly (1.5 is a bf16 number), zero queries give the column mean
+    vc = torch.full_like(v, 1.5)
+    assert (capi.forward(q.to(gpu), k.to(gpu), vc.to(gpu), H).float() == 1.5).all()
+    zq = capi.forward(torch.zeros_like(q).to(gpu), k.to(gpu), v.to(gpu), H)
+    want = v.double().mean(dim=1, keepdim=True).float().expand(B, L, R * H)
+    assert _max_err(zq, want) <= 2e-3
+    with pytest.raises(TypeError):
+        capi.forward(q.to(gpu), k.half().to(gpu), v.to(gpu), H)
+
+
 def test_causal_with_mask_is_rejected(gpu):
     x = torch.zeros(1, 64, 64, dtype=torch.float16, device=gpu)
     m = torch.zeros(1, 64, 64, dtype=torch.float16, device=gpu)
