@@ -5,17 +5,22 @@
 // reference's attention_kernel and every threadblock_* helper it calls
 // (reference include/fused_attn.cuh:48-538 and :605-858).
 //
+// Two kernels share the pieces in this file and in fused_attn_kernel_impl.inc:
+//   fwd_kernel           four waves, software pipelined inside each wave; also the additive-mask
+//                        variant and the causal variant for small grids
+//   fwd_kernel_pingpong  eight waves in two groups that alternate vector and matrix phases;
+//                        plain and causal
 // Work decomposition
-//   workgroup  = NW wave64s, each wave owns 64 query rows (two 32-row blocks)
-//   K/V        = streamed in BK-key tiles, global -> registers -> LDS, double buffered
-//   per 32 keys: S^T = K_sub * Q^T        v_mfma_f32_32x32x16_f16, Q held in registers
+//   workgroup  = NW wave64s, each wave owns 32 NQB query rows (NQB = 1 or 2 blocks of 32)
+//   K/V        = streamed in 64-key tiles, global -> registers -> LDS ring (2 or 3 slots)
+//   per 32 keys: S^T = K_sub * Q^T        v_mfma_f32_32x32x16_{f16,bf16}, Q held in registers
 //                online softmax on S^T     f32, state (m, l) per lane
 //                O^T += V_sub^T * P^T      same MFMA, V^T fetched with ds_read_b64_tr_b16
 //
 // Why the transposed products: in the 32x32 accumulator layout lane l owns column
 // (l % 32) -- one query -- and 16 of the 32 rows (keys); lane l^32 owns the other 16.
 // A softmax row therefore lives in one lane pair, so row max / row sum need 15 in-lane
-// ops and a single v_permlane32_swap.  The f16-packed P^T registers are, as they stand,
+// ops and a single v_permlane32_swap.  The packed 16-bit P^T registers are, as they stand,
 // a valid B operand of the second product provided the A operand (V^T) enumerates keys
 // in the same order, which the transpose-read from a row-major V tile provides.
 //
