@@ -201,6 +201,32 @@ def test_heads_and_batches_are_independent_bitwise(gpu):
     assert not torch.equal(out[0, :, H:2 * H], base[0, :, H:2 * H])
 
 
+def test_launch_can_be_captured_in_a_graph_and_replayed(gpu):
+    # The library allocates nothing and clears nothing at launch time, so a launch on a capturing
+    # stream is recorded as a single kernel node.  Replays must follow the contents of the (static)
+    # input buffers and agree bitwise with eager launches, with eager work between the replays.
+    import fused_attn
+
+    B, R, L, H = 2, 16, 1024, 64
+    q, k, v = (_rand((B, L, R * H), 2400 + i).to(gpu) for i in range(3))
+    eager0 = fused_attn.attention_forward(H, 64, q, k, v)        # also the warm-up launch
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = fused_attn.attention_forward(H, 64, q, k, v)
+    for rep in range(4):
+        if rep:
+            q.copy_(_rand((B, L, R * H), 2410 + rep))            # new inputs in the captured buffers
+        eager = fused_attn.attention_forward(H, 64, q, k, v)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        if rep == 0:
+            assert torch.equal(out, eager0)
+    want = attention(q.cpu(), k.cpu(), v.cpu(), H)
+    assert _max_err(out, want) <= TOL
+
+
 # ---- additive mask ---------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("L,H,offset", [(64, 64, 0), (200, 32, 0), (300, 128, 0), (203, 64, 0), (97, 16, 0),
