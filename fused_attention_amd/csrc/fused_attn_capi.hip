@@ -15,8 +15,7 @@ namespace {
 constexpr int kKeyTile = 64;     // keys per LDS tile
 constexpr int kNumCu = 256;      // compute units of one MI355X
 
-// Launch shape: wave64s per workgroup, blocks of 32 query rows per wave, waves per SIMD the
-// registers are budgeted for.
+// Launch shape: wave64s per workgroup and blocks of 32 query rows per wave.
 struct Shape {
     int waves;
     int nqb;

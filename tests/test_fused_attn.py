@@ -377,16 +377,31 @@ def test_causal_on_large_grids(gpu, B, R, L, H):
         assert ((lse[b, h].cpu() - want).abs() / (1 + want.abs())).max().item() <= 1e-3
 
 
-@pytest.mark.parametrize("B,R,L,H", [(8, 64, 512, 64), (4, 40, 700, 128), (16, 40, 384, 16)])
+@pytest.mark.parametrize("B,R,L,H", [
+    (8, 64, 512, 64), (16, 40, 384, 16), (2, 64, 1024, 32),     # 8-byte mask loads
+    (2, 64, 1023, 64),                                           # element-wise mask loads, ragged end
+    (4, 40, 700, 128),
+])
 def test_additive_mask_on_large_grids(gpu, B, R, L, H):
     q, k, v = (_rand((B, L, R * H), 3970 + L + i) for i in range(3))
     g = torch.Generator().manual_seed(3975)
     mask = torch.where(torch.rand(B, L, L, generator=g) < 0.3, float("-inf"), 0.0)
     mask = (mask + torch.randn(B, L, L, generator=g) * 0.5).to(torch.float16)
     mask[:, :, 0] = 0
+    mask[0, 5] = float("-inf")                  # two fully masked rows: zeros, not NaN
+    mask[B - 1, L - 1] = float("-inf")
     got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, mask=mask.to(gpu))
     assert torch.isfinite(got.float()).all()
-    _check_pairs(got, q, k, v, H, [(0, 0), (B // 2, R // 2), (B - 1, R - 1)], mask=mask.float())
+    assert (got[0, 5] == 0).all() and (got[B - 1, L - 1] == 0).all()
+    mask[0, 5] = 0                              # the oracle would give NaN there; compare the other rows
+    mask[B - 1, L - 1] = 0
+    keep = torch.ones(B, L, dtype=torch.bool)
+    keep[0, 5] = keep[B - 1, L - 1] = False
+    for b, h in [(0, 0), (B // 2, R // 2), (B - 1, R - 1)]:
+        sl = slice(h * H, (h + 1) * H)
+        want = attention(q[b:b + 1, :, sl], k[b:b + 1, :, sl], v[b:b + 1, :, sl], H, mask=mask[b:b + 1].float())
+        err = (got[b, :, sl].float().cpu() - want[0]).abs()
+        assert err[keep[b]].max().item() <= TOL, (b, h)
 
 
 # ---- bfloat16 inputs (FA_FLAG_BF16) ------------------------------------------------------------------
