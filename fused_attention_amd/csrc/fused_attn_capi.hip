@@ -28,8 +28,7 @@ struct Shape {
 //   {4, 2}  four 64-row waves, 256 queries per workgroup, two resident per compute unit;
 //   {4, 1}  four 32-row waves, 128 queries per workgroup, three (head_dim <= 64) or two
 //           (head_dim 128) resident per compute unit: more, smaller workgroups for small problems.
-// head_dim 128 with 64-row waves needs the whole register file of a SIMD for one wave, and the
-// additive-mask variant exists only with four waves.
+// head_dim 128 with 64-row waves needs the whole register file of a SIMD for one wave.
 int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // How well a shape uses the chip, in 1/1024: the share of the (rounds x slots) grid of resident
@@ -43,11 +42,9 @@ int64_t usage(int64_t heads, int64_t L, int64_t rows, int64_t slots) {
 
 Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask, bool causal) {
     const int64_t heads = B * R;
-    // the additive-mask variant exists only with four waves
-    if (has_mask) {
-        if (H > 64) return {4, 1};
-        return heads * ceil_div(L, 256) >= 2 * kNumCu ? Shape{4, 2} : Shape{4, 1};
-    }
+    // the additive-mask variant exists only with four 32-row waves (the mask staging registers and
+    // LDS slabs leave room for two such workgroups per compute unit, not for 64-row waves)
+    if (has_mask) return {4, 1};
     // The ping-pong kernel is the fastest per compute unit, so it is taken whenever its
     // workgroups fill the chip well enough.  Thresholds measured on MI355X: a lone round may be
     // emptier than the tail of several, because idle units leave the busy ones more of the
@@ -82,7 +79,7 @@ hipError_t allow_large_lds(const void* kernel, int bytes) {
 // BF selects the bf16 instantiation (namespace fa::bf16) of the same kernel source.
 template <int H, int NW, int NQB, int WPE, int MODE, bool BF>
 hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
-    constexpr int lds = fa::lds_bytes<H, NW, kKeyTile>();
+    constexpr int lds = MODE == fa::kAdditive ? fa::lds_bytes_masked<H, NW, kKeyTile, NQB>() : fa::lds_bytes<H, NW, kKeyTile>();
     auto kernel = BF ? fa::bf16::fwd_kernel<H, NW, kKeyTile, NQB, WPE, MODE> : fa::fwd_kernel<H, NW, kKeyTile, NQB, WPE, MODE>;
     if constexpr (lds > 64 * 1024) {
         const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), lds);
@@ -118,7 +115,7 @@ hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) 
         }
     }
     // four waves: 64-row waves where the registers allow it
-    if constexpr (H > 64)
+    if constexpr (H > 64 || MODE == fa::kAdditive)
         return launch<H, 4, 1, 2, MODE, BF>(p, stream);
     else
         return sh.nqb == 2 ? launch<H, 4, 2, 2, MODE, BF>(p, stream) : launch<H, 4, 1, 3, MODE, BF>(p, stream);

@@ -89,6 +89,18 @@ constexpr int lds_bytes() {
     return 2 * BK * (G::KSTR + G::VSTR) * (int)sizeof(_Float16);
 }
 
+// Additive-mask variant: behind the K/V buffers every wave has a private slab for the mask values
+// of its 32 NQB queries and the 64 keys of the current tile (row stride kMaskStr halves: 128 bytes
+// of mask plus 16 of padding).
+constexpr int kMaskStr = 72;
+// Not at head_dim 128: there the slabs would cost the second resident workgroup of a compute unit.
+template <int H>
+constexpr bool mask_staging() { return H <= 64; }
+template <int H, int NW, int BK, int NQB>
+constexpr int lds_bytes_masked() {
+    return lds_bytes<H, NW, BK>() + (mask_staging<H>() ? NW * 32 * NQB * kMaskStr * (int)sizeof(_Float16) : 0);
+}
+
 // NaN-propagating maximum: lowers to v_maximum3_f32 without the input canonicalisation that
 // fmaxf needs in IEEE mode.
 __device__ __forceinline__ float fmax2(float a, float b) { return __builtin_elementwise_maximum(a, b); }
