@@ -40,11 +40,14 @@ int64_t usage(int64_t heads, int64_t L, int64_t rows, int64_t slots) {
     return wgs * L * 1024 / (ceil_div(wgs, slots) * slots * per_head * rows);
 }
 
-Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask, bool causal) {
+// mask_rows_aligned: an additive mask whose rows are 16-byte aligned (L % 8 == 0, aligned pointer).
+Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask, bool mask_rows_aligned,
+                 bool causal) {
     const int64_t heads = B * R;
-    // the additive-mask variant exists only with four 32-row waves (the mask staging registers and
-    // LDS slabs leave room for two such workgroups per compute unit, not for 64-row waves)
-    if (has_mask) return {4, 1};
+    // The ping-pong kernel takes an additive mask only through its coalesced, LDS-staged fetch;
+    // any other mask goes to four 32-row waves (the mask staging registers and LDS slabs leave room
+    // for two such workgroups per compute unit, not for 64-row waves).
+    if (has_mask && !mask_rows_aligned) return {4, 1};
     // The ping-pong kernel is the fastest per compute unit, so it is taken whenever its
     // workgroups fill the chip well enough.  Thresholds measured on MI355X: a lone round may be
     // emptier than the tail of several, because idle units leave the busy ones more of the
@@ -55,6 +58,7 @@ Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask, bool
     const bool pingpong = wgs8 >= 2 * kNumCu ? usage8 >= 614 : usage8 >= (wgs8 <= kNumCu ? 614 : 717);
     if (H > 64) return pingpong ? Shape{8, 1} : Shape{4, 1};
     if (pingpong) return {8, 2};
+    if (has_mask) return {4, 1};
     // everything resident at once: the smallest workgroups give the most parallelism
     if (heads * ceil_div(L, 128) <= 3 * kNumCu) return {4, 1};
     return usage(heads, L, 256, 2 * kNumCu) > usage(heads, L, 128, 3 * kNumCu) ? Shape{4, 2} : Shape{4, 1};
@@ -90,10 +94,10 @@ hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
-template <int H, int NW, int NQB, int WPE, bool CAUSAL, bool BF>
+template <int H, int NW, int NQB, int WPE, int MODE, bool BF>
 hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
-    constexpr int lds = fa::lds_bytes_pingpong<H, NQB>();
-    auto kernel = BF ? fa::bf16::fwd_kernel_pingpong<H, NW, NQB, WPE, CAUSAL> : fa::fwd_kernel_pingpong<H, NW, NQB, WPE, CAUSAL>;
+    constexpr int lds = MODE == fa::kAdditive ? fa::lds_bytes_pingpong_masked<H, NW, NQB>() : fa::lds_bytes_pingpong<H, NQB>();
+    auto kernel = BF ? fa::bf16::fwd_kernel_pingpong<H, NW, NQB, WPE, MODE> : fa::fwd_kernel_pingpong<H, NW, NQB, WPE, MODE>;
     if constexpr (lds > 64 * 1024) {
         const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), lds);
         if (e != hipSuccess) return e;
@@ -105,14 +109,12 @@ hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
 
 template <int H, int MODE, bool BF>
 hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) {
-    if constexpr (MODE != fa::kAdditive) {
-        // plain and causal: the ping-pong kernel for the eight-wave shapes
-        if (sh.waves == 8) {
-            if constexpr (H > 64)
-                return launch_pingpong<H, 8, 1, 2, MODE == fa::kCausal, BF>(p, stream);
-            else
-                return launch_pingpong<H, 8, 2, 2, MODE == fa::kCausal, BF>(p, stream);
-        }
+    // the ping-pong kernel for the eight-wave shapes
+    if (sh.waves == 8) {
+        if constexpr (H > 64)
+            return launch_pingpong<H, 8, 1, 2, MODE, BF>(p, stream);
+        else
+            return launch_pingpong<H, 8, 2, 2, MODE, BF>(p, stream);
     }
     // four waves: 64-row waves where the registers allow it
     if constexpr (H > 64 || MODE == fa::kAdditive)
@@ -153,7 +155,8 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     if (L > kMaxInt - 4096 || B > kMaxInt || R > kMaxInt) return FA_ERR_TOO_LARGE;
     // the tile loaders keep 32-bit byte offsets inside a 64-key tile
     if (stride_l > ((int64_t)1 << 24)) return FA_ERR_TOO_LARGE;
-    *shape = pick_shape(B, R, L, H, mask != nullptr, causal);
+    *shape = pick_shape(B, R, L, H, mask != nullptr,
+                        (L % 8) == 0 && (reinterpret_cast<uintptr_t>(mask) & 15u) == 0, causal);
     const int64_t bq = shape->rows();
     int64_t n_qtiles = (L + bq - 1) / bq;
     if (causal && shape->waves == 8) n_qtiles = (n_qtiles + 1) / 2;   // pairs of query tiles

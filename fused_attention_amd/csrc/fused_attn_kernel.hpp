@@ -239,6 +239,15 @@ constexpr int lds_bytes_pingpong() {
     return 3 * 64 * (G::KSTR + G::VSTR) * (int)sizeof(_Float16);
 }
 
+// Additive-mask variant of the ping-pong kernel: behind the rings every wave has a private slab
+// for the mask values of its 32 NQB queries and the 32 keys of one sub-tile (row stride
+// kMaskSubStr halves: 64 bytes of mask plus 16 of padding).
+constexpr int kMaskSubStr = 40;
+template <int H, int NW, int NQB>
+constexpr int lds_bytes_pingpong_masked() {
+    return lds_bytes_pingpong<H, NQB>() + NW * 32 * NQB * kMaskSubStr * (int)sizeof(_Float16);
+}
+
 __device__ __forceinline__ void phase_barrier() {
     // LDS traffic of this wave is complete (writes visible, reads returned) before the barrier;
     // global loads in flight are deliberately not waited for.  The scheduling barriers keep the

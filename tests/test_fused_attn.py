@@ -307,6 +307,13 @@ def test_lse_of_the_pingpong_kernel(gpu):
 
 # ---- every launch shape, plain and masked -------------------------------------------------------------
 
+def _check_pairs_tol(got, q, k, v, H, pairs, mask, tol):
+    for b, h in pairs:
+        sl = slice(h * H, (h + 1) * H)
+        want = attention(q[b:b + 1, :, sl], k[b:b + 1, :, sl], v[b:b + 1, :, sl], H, mask=mask[b:b + 1])
+        assert _max_err(got[b:b + 1, :, sl], want) <= tol, (b, h)
+
+
 def _check_pairs(got, q, k, v, H, pairs, mask=None):
     """Compares the listed (batch, head) slices of a full-tensor result against the oracle."""
     for b, h in pairs:
@@ -378,9 +385,10 @@ def test_causal_on_large_grids(gpu, B, R, L, H):
 
 
 @pytest.mark.parametrize("B,R,L,H", [
-    (8, 64, 512, 64), (16, 40, 384, 16), (2, 64, 1024, 32),     # 8-byte mask loads
-    (2, 64, 1023, 64),                                           # element-wise mask loads, ragged end
-    (4, 40, 700, 128),
+    (8, 64, 512, 64), (16, 40, 384, 16), (2, 64, 1024, 32),     # eight-wave kernel, mask staged through LDS
+    (4, 40, 704, 128),                                           # ... head_dim 128, ragged end
+    (2, 64, 1023, 64),                                           # element-wise mask loads (L % 4 != 0)
+    (4, 40, 700, 128),                                           # 8-byte mask loads (L % 8 != 0)
 ])
 def test_additive_mask_on_large_grids(gpu, B, R, L, H):
     q, k, v = (_rand((B, L, R * H), 3970 + L + i) for i in range(3))
@@ -430,15 +438,15 @@ def test_bf16_inputs(gpu, B, R, L, H, causal):
         assert ((lse[b, h].cpu() - want_lse).abs() / (1 + want_lse.abs())).max().item() <= 2e-3
 
 
-def test_bf16_additive_mask_and_closed_forms(gpu):
-    B, R, L, H = 2, 2, 200, 64
+@pytest.mark.parametrize("B,R,L,H", [(2, 2, 200, 64), (8, 64, 512, 64)])
+def test_bf16_additive_mask_and_closed_forms(gpu, B, R, L, H):
     q, k, v = (_rand((B, L, R * H), 4300 + i).to(torch.bfloat16) for i in range(3))
     g = torch.Generator().manual_seed(4310)
     mask = torch.where(torch.rand(B, L, L, generator=g) < 0.3, float("-inf"), 0.0)
     mask = (mask + torch.randn(B, L, L, generator=g) * 0.5).to(torch.bfloat16)
     mask[:, :, 0] = 0
     got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, mask=mask.to(gpu))
-    assert _max_err(got, attention(q, k, v, H, mask=mask)) <= BF16_TOL
+    _check_pairs_tol(got, q, k, v, H, [(0, 0), (B - 1, R - 1)], mask.float(), BF16_TOL)
     # constant V comes back exactly (1.5 is a bf16 number), zero queries give the column mean
     vc = torch.full_like(v, 1.5)
     assert (capi.forward(q.to(gpu), k.to(gpu), vc.to(gpu), H).float() == 1.5).all()
