@@ -6,10 +6,10 @@
 // (reference include/fused_attn.cuh:48-538 and :605-858).
 //
 // Two kernels share the pieces in this file and in fused_attn_kernel_impl.inc:
-//   fwd_kernel           four waves, software pipelined inside each wave; also the additive-mask
-//                        variant and the causal variant for small grids
+//   fwd_kernel           four waves, software pipelined inside each wave; its additive-mask and
+//                        causal variants (plain loop) serve small grids and unaligned masks
 //   fwd_kernel_pingpong  eight waves in two groups that alternate vector and matrix phases;
-//                        plain and causal
+//                        plain, causal and additive mask (mask rows 16-byte aligned)
 // Work decomposition
 //   workgroup  = NW wave64s, each wave owns 32 NQB query rows (NQB = 1 or 2 blocks of 32)
 //   K/V        = streamed in 64-key tiles, global -> registers -> LDS ring (2 or 3 slots)
