@@ -6,8 +6,8 @@
 // (reference include/fused_attn.cuh:48-538 and :605-858).
 //
 // Two kernels share the pieces in this file and in fused_attn_kernel_impl.inc:
-//   fwd_kernel           four waves, software pipelined inside each wave; its additive-mask and
-//                        causal variants (plain loop) serve small grids and unaligned masks
+//   fwd_kernel           four waves, software pipelined inside each wave (plain and causal); its
+//                        additive-mask variant (plain loop) serves small grids and unaligned masks
 //   fwd_kernel_pingpong  eight waves in two groups that alternate vector and matrix phases;
 //                        plain, causal and additive mask (mask rows 16-byte aligned)
 // Work decomposition
