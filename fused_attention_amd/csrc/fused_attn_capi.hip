@@ -37,7 +37,10 @@ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 int64_t usage(int64_t heads, int64_t L, int64_t rows, int64_t slots) {
     const int64_t per_head = ceil_div(L, rows);
     const int64_t wgs = heads * per_head;
-    return wgs * L * 1024 / (ceil_div(wgs, slots) * slots * per_head * rows);
+    // in floating point: the products overflow 64 bits for the largest accepted shapes
+    const double filled = (double)wgs / ((double)ceil_div(wgs, slots) * (double)slots);
+    const double rows_used = (double)L / ((double)per_head * (double)rows);
+    return (int64_t)(1024.0 * filled * rows_used);
 }
 
 // mask_rows_aligned: an additive mask whose rows are 16-byte aligned (L % 8 == 0, aligned pointer).
@@ -152,7 +155,7 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return FA_ERR_MISALIGNED;
     if (mask != nullptr && (reinterpret_cast<uintptr_t>(mask) & 1u) != 0) return FA_ERR_MISALIGNED;
     constexpr int64_t kMaxInt = 0x7fffffff;
-    if (L > kMaxInt - 4096 || B > kMaxInt || R > kMaxInt) return FA_ERR_TOO_LARGE;
+    if (L > kMaxInt - 4096 || B > kMaxInt || R > kMaxInt || B * R > kMaxInt) return FA_ERR_TOO_LARGE;
     // the tile loaders keep 32-bit byte offsets inside a 64-key tile
     if (stride_l > ((int64_t)1 << 24)) return FA_ERR_TOO_LARGE;
     *shape = pick_shape(B, R, L, H, mask != nullptr,
