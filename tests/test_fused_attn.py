@@ -103,6 +103,37 @@ def test_config_c4_sampled_heads(gpu):
     assert (got[sel] - want[sel]).abs().max().item() <= TOL
 
 
+def test_full_size_properties_without_an_oracle(gpu):
+    # Size-independent properties at the headline size: the output is linear in V, and a constant
+    # shift of all values shifts the output by the same constant (the weights of a row sum to one).
+    import fused_attn
+
+    w = workloads.WORKLOADS["c3"]
+    q, k, v = (t.to(gpu) for t in workloads.make_inputs(w))
+    g = torch.Generator().manual_seed(97)
+    v2 = (torch.randn(v.shape, generator=g) * 0.5).to(torch.float16).to(gpu)
+    o1 = fused_attn.attention_forward(w.H, 64, q, k, v).float()
+    o2 = fused_attn.attention_forward(w.H, 64, q, k, v2).float()
+    vsum = (v.float() + 2.0 * v2.float()).half()
+    o12 = fused_attn.attention_forward(w.H, 64, q, k, vsum).float()
+    # fp16 rounding of the summed values and of the three outputs: a few 1e-3
+    assert (o12 - (o1 + 2.0 * o2)).abs().max().item() <= TOL
+    shifted = fused_attn.attention_forward(w.H, 64, q, k, (v.float() + 1.0).half()).float()
+    assert (shifted - (o1 + 1.0)).abs().max().item() <= TOL
+
+
+def test_duplicated_keys_at_long_sequence(gpu):
+    # Concatenating (K, V) with itself leaves the output unchanged: 8192 -> 16384 keys at head_dim
+    # 128 crosses from one launch shape to another and doubles the number of key tiles.
+    B, R, L, H = 1, 32, 8192, 128
+    q, k, v = (_rand((B, L, R * H), 5100 + i, std=0.5).to(gpu) for i in range(3))
+    once = capi.forward(q, k, v, H).float()
+    q2 = torch.cat([q, q], dim=1)
+    twice = capi.forward(q2, torch.cat([k, k], dim=1), torch.cat([v, v], dim=1), H).float()
+    assert (twice[:, :L] - once).abs().max().item() <= 2e-3
+    assert (twice[:, L:] - once).abs().max().item() <= 2e-3
+
+
 # ---- shapes the reference never exercised ---------------------------------------------------------
 
 @pytest.mark.parametrize("B,R,L,H", [
