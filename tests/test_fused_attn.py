@@ -258,6 +258,51 @@ def test_launch_can_be_captured_in_a_graph_and_replayed(gpu):
     assert _max_err(out, want) <= TOL
 
 
+def _random_cases(n, seed):
+    import random
+
+    rng = random.Random(seed)
+    cases = []
+    for i in range(n):
+        H = rng.choice([16, 32, 64, 128])
+        L = rng.choice([rng.randint(1, 96), rng.randint(97, 700), rng.randint(701, 2600)])
+        heads = rng.choice([1, 3, 8, 24, 96, 300])
+        B = rng.choice([1, 2, 3])
+        R = max(1, heads // B)
+        if B * R * L * H > 40_000_000:
+            R = max(1, 40_000_000 // (B * L * H))
+        mode = rng.choice(["plain", "plain", "causal", "mask"])
+        cases.append((i, B, R, L, H, mode))
+    return cases
+
+
+@pytest.mark.parametrize("i,B,R,L,H,mode", _random_cases(28, 20261125))
+def test_seeded_random_shapes(gpu, i, B, R, L, H, mode):
+    # shapes drawn once from a fixed seed: odd lengths, every head_dim, grids from one workgroup to
+    # several rounds of the chip, all three modes
+    q, k, v = (_rand((B, L, R * H), 6000 + 3 * i + j) for j in range(3))
+    mask = None
+    dev_mask = None
+    if mode == "causal":
+        mask = causal_mask(B, L)
+    elif mode == "mask":
+        g = torch.Generator().manual_seed(6100 + i)
+        mask = torch.where(torch.rand(B, L, L, generator=g) < 0.25, float("-inf"), 0.0)
+        mask = (mask + torch.randn(B, L, L, generator=g) * 0.5).to(torch.float16)
+        mask[:, :, 0] = 0
+        dev_mask = mask.to(gpu)
+        mask = mask.float()
+    got, lse = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, mask=dev_mask, causal=(mode == "causal"),
+                            return_lse=True)
+    assert torch.isfinite(got.float()).all()
+    pairs = sorted({(0, 0), (B - 1, R // 2), (B - 1, R - 1)})
+    _check_pairs(got, q, k, v, H, pairs, mask=mask)
+    for b, h in pairs:
+        sl = slice(h * H, (h + 1) * H)
+        want = attention_lse(q[b:b + 1, :, sl], k[b:b + 1, :, sl], H, mask=None if mask is None else mask[b:b + 1])[0, 0]
+        assert ((lse[b, h].cpu() - want).abs() / (1 + want.abs())).max().item() <= 1e-3
+
+
 # ---- additive mask ---------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("L,H,offset", [(64, 64, 0), (200, 32, 0), (300, 128, 0), (203, 64, 0), (97, 16, 0),
