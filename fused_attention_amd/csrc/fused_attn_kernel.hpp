@@ -233,10 +233,33 @@ __device__ __forceinline__ const _Float16* v_operand_ptr(const _Float16* vs, int
            4 * (s16 & 3);
 }
 
+// Ring tiles of the ping-pong kernel are chunk-major: a 64-key tile of H columns is stored as H / 8
+// columns of 64 rows x 16 bytes, column c at c * kColStride halves.  One direct-to-LDS load of a
+// wave (64 lanes x 16 bytes, contiguous in LDS) fills one column, lane = key row.  The 64-byte pad
+// between columns spreads the four columns touched by a transpose read over all banks.
+constexpr int kColStride = 64 * 8 + 32;
+template <int H>
+constexpr int ring_tile_k() { return (H / 8) * kColStride; }
+template <int H>
+constexpr int ring_tile_v() { return (Geometry<H>::HV / 8) * kColStride; }
+// Per-lane part of the K operand address in a ring tile: row (sub * 32 + lane % 32) of column
+// lane / 32; k-step kk adds 2 kk columns.
+__device__ __forceinline__ const _Float16* k_ring_ptr(const _Float16* ks, int sub, int lane) {
+    return ks + (lane >> 5) * kColStride + (sub * 32 + (lane & 31)) * 8;
+}
+
+// Per-lane part of the transpose-read address in a ring tile (see v_operand_ptr for which element
+// ends up where): lane s of a 16-lane group points at row key0 + s / 4, halves 4 (s % 4) ... of the
+// 32-byte span that starts at column 2 * ((lane / 16) % 2); head-dim block db adds 4 db columns.
+__device__ __forceinline__ const _Float16* v_ring_ptr(const _Float16* vs, int sub, int lane) {
+    const int s16 = lane & 15;
+    return vs + (2 * ((lane >> 4) & 1) + ((s16 & 3) >> 1)) * kColStride +
+           (sub * 32 + 4 * (lane >> 5) + (s16 >> 2)) * 8 + 4 * (s16 & 1);
+}
+
 template <int H, int NQB>
 constexpr int lds_bytes_pingpong() {
-    using G = Geometry<H>;
-    return 3 * 64 * (G::KSTR + G::VSTR) * (int)sizeof(_Float16);
+    return 3 * (ring_tile_k<H>() + ring_tile_v<H>()) * (int)sizeof(_Float16);
 }
 
 // Additive-mask variant of the ping-pong kernel: behind the rings every wave has a private slab
@@ -258,54 +281,49 @@ __device__ __forceinline__ void phase_barrier() {
     __builtin_amdgcn_sched_barrier(0);
 }
 
-// One group's share of a 64-key tile: per-thread chunk offsets are computed once, a tile is then
-// fetched with one pointer bump and NP 16-byte loads.
-template <int H, int NT>
-struct GroupLoader {
+// One group's share of a 64-key ring tile, fetched straight into LDS.  Wave w of the group (NWG
+// waves) owns the columns w * NP ... w * NP + NP - 1; lane l fetches the 16 bytes of key row l.
+// Rows at or beyond L are read from row L - 1 instead: their scores are masked to -inf, or belong
+// to sub-tiles that are never consumed, and a probability of exactly zero times a finite V row
+// contributes nothing.  Tiles starting at or beyond `limit` are not fetched at all (limit <= L).
+// The loads are asynchronous: the issuing wave waits for vmcnt before the barrier that hands the
+// tile to its readers.
+template <int H, int NWG>
+struct RingLoader {
     static constexpr int CPR = H / 8;
-    static constexpr int NCHUNK = 64 * CPR;
-    static constexpr int NP = (NCHUNK + NT - 1) / NT;
-    static constexpr bool EXACT = NCHUNK % NT == 0;
-    u32x4 reg[NP];
-    int64_t goff[NP];   // element offset of the chunk inside a tile
-    int loff[NP];       // element offset of the chunk inside an LDS tile
-    int row[NP];
-    int col[NP];
+    static constexpr int NP = (CPR + NWG - 1) / NWG;
+    int col0;
+    uint32_t lane_off;   // byte offset of this lane's row inside a full tile
 
-    __device__ __forceinline__ void init(int64_t stride_l, int lds_stride, int gtid) {
-#pragma unroll
-        for (int i = 0; i < NP; ++i) {
-            const int idx = gtid + i * NT;
-            row[i] = (EXACT || idx < NCHUNK) ? idx / CPR : (1 << 30);
-            col[i] = (idx % CPR) * 8;
-            goff[i] = (int64_t)(idx / CPR) * stride_l + (idx % CPR) * 8;
-            loff[i] = (idx / CPR) * lds_stride + (idx % CPR) * 8;
-        }
+    __device__ __forceinline__ void init(int wave_in_group, int64_t stride_l, int lane) {
+        col0 = wave_in_group * NP;
+        lane_off = (uint32_t)lane * (uint32_t)stride_l * 2u;
     }
-    // Rows at or beyond L are read from row L - 1 instead (no predicated loads, so no load ever
-    // waits for another): their scores are masked to -inf, or belong to sub-tiles that are never
-    // consumed, and a probability of exactly zero times a finite V row contributes nothing.
-    // Tiles starting at or beyond `limit` are not fetched at all (limit <= L).
-    __device__ __forceinline__ void load(const _Float16* src, int64_t stride_l, int key0, int limit, int L) {
+    // The load is written in assembly so that the compiler does not see an LDS write: it would
+    // otherwise wait for the load before the next LDS read of the wave.  M0 holds the LDS address
+    // of lane 0's 16 bytes; lane l lands 16 l bytes further on.
+    static __device__ __forceinline__ void dma16(uint32_t lds_addr, const _Float16* base, uint32_t voff) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :: "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
+    }
+    __device__ __forceinline__ void issue(const _Float16* src, int64_t stride_l, int key0, int limit, int L,
+                                          _Float16* tile, int lane) const {
+        issue_at(src + (int64_t)key0 * stride_l + col0 * 8, stride_l, key0, limit, L, tile, lane);
+    }
+    // `base` = src + key0 * stride_l + 8 * col0, kept by callers that walk the tiles in order
+    __device__ __forceinline__ void issue_at(const _Float16* base, int64_t stride_l, int key0, int limit, int L,
+                                             _Float16* tile, int lane) const {
         if (key0 >= limit) return;
-        if (key0 + 64 <= L && EXACT) {
-            const _Float16* tile = src + (int64_t)key0 * stride_l;
-#pragma unroll
-            for (int i = 0; i < NP; ++i) reg[i] = *reinterpret_cast<const u32x4*>(tile + goff[i]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < NP; ++i) {
-                const int r = min(key0 + min(row[i], 63), L - 1);
-                reg[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)r * stride_l + col[i]);
-            }
-        }
-    }
-    __device__ __forceinline__ void store(_Float16* dst) const {
+        uint32_t voff = lane_off;
+        if (key0 + 64 > L) voff = (uint32_t)(min(key0 + lane, L - 1) - key0) * (uint32_t)stride_l * 2u;
+        const uint32_t lds0 = (uint32_t)(uintptr_t)(FA_LDS void*)tile + (uint32_t)col0 * (kColStride * 2);
 #pragma unroll
         for (int i = 0; i < NP; ++i)
-            if (EXACT || row[i] < 64) *reinterpret_cast<u32x4*>(dst + loff[i]) = reg[i];
+            if (CPR % NWG == 0 || col0 + i < CPR) dma16(lds0 + i * (kColStride * 2), base + i * 8, voff);
     }
 };
+
+__device__ __forceinline__ void wait_ring_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 }  // namespace fa
 
