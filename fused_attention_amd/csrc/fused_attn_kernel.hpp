@@ -192,9 +192,12 @@ struct TileLoader {
 // Largest partial row sum (16 terms) the fast path of the online softmax accepts.
 constexpr float kTrip = 16384.f;
 
-// Eight-wave kernel: bias (log2 units) of the reference the exponentials are taken against, and the
-// bits of a packed pair of 16-bit floats (fp16 or bf16: 2.0 is 0x4000 in both) that say "2.0 or more".
+// Eight-wave kernel: bias (log2 units) of the reference the exponentials are taken against, and what
+// its fast path accepts: with 64-row waves the largest sum of a query's 32 probabilities of one
+// sub-tile, with 32-row waves no packed pair of 16-bit floats (fp16 or bf16: 2.0 is 0x4000 in both)
+// with the "2.0 or more" bit set.
 constexpr float kBias = 6.0f;
+constexpr float kTripSum = 32768.f;
 constexpr uint32_t kTripBits = 0x40004000u;
 __device__ __forceinline__ bool trips(uint32_t orv) { return (orv & kTripBits) != 0u; }
 
@@ -271,12 +274,14 @@ constexpr int lds_bytes_pingpong_masked() {
     return lds_bytes_pingpong<H, NQB>() + NW * 32 * NQB * kMaskSubStr * (int)sizeof(_Float16);
 }
 
-__device__ __forceinline__ void phase_barrier() {
-    // LDS traffic of this wave is complete (writes visible, reads returned) before the barrier;
-    // global loads in flight are deliberately not waited for.  The scheduling barriers keep the
-    // compiler from moving matrix or vector instructions of one phase into the next.
+// Barrier between the phases of the ping-pong kernel.  It does not wait for the wave's own LDS
+// reads: nothing is handed from wave to wave through LDS stores (the rings are written by
+// direct-to-LDS loads, which their issuer waits for with vmcnt), and every read of a ring slot is
+// consumed by a matrix instruction at least one barrier before the loads that overwrite the slot
+// are issued.  The scheduling barriers keep the compiler from moving matrix or vector
+// instructions of one phase into the next.
+__device__ __forceinline__ void ring_barrier() {
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
 }
