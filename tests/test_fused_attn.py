@@ -439,6 +439,29 @@ def test_eight_wave_kernel_on_adversarial_scores(gpu, B, R, L, H, kind):
     assert scores.abs().max() > 20
 
 
+@pytest.mark.parametrize("B,R,L,H", [(2, 16, 4096, 64), (2, 64, 1024, 128)])
+@pytest.mark.parametrize("step_log2", [6.5, 14.0, 15.5, 16.5, 18.0, 21.0, 22.5, 26.0])
+def test_eight_wave_kernel_reference_lag(gpu, B, R, L, H, step_log2):
+    # All scores are 0 up to key 96 and jump by step_log2 (in units of log2) from there on, so the
+    # reference the kernel took from the first keys lags by exactly that much: probabilities taken
+    # against it land below, inside and beyond the window in which the fp16 pack saturates at 65504
+    # instead of overflowing to inf (the check must catch those too).  With the jump the first 96
+    # keys carry a weight of 2^-step each, so the output is the mean of V over keys 96.. to within
+    # that weight.
+    q = torch.zeros(B, L, R * H)
+    k = torch.zeros(B, L, R * H)
+    q[:, :, ::H] = math.sqrt(H)                       # component 0 of every head: raw score = sqrt(H) * k0
+    k[:, 96:, ::H] = step_log2 / math.log2(math.e)    # scaled score in natural-log units
+    q, k = q.half(), k.half()
+    v = _rand((B, L, R * H), 4300 + L)
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H)
+    assert torch.isfinite(got.float()).all()
+    _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R - 1)])
+    if step_log2 >= 14:
+        want = v[:, 96:].float().mean(dim=1, keepdim=True)
+        assert (got.float().cpu() - want).abs().max().item() <= 5e-3
+
+
 @pytest.mark.parametrize("B,R,L,H", [
     (4, 16, 4096, 64),      # eight-wave workgroups, each taking a pair of query tiles (8 tiles per head)
     (2, 64, 1300, 64),      # ... with an odd number of tiles (the middle one runs alone) and a ragged end
