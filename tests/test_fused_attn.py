@@ -276,7 +276,22 @@ def _random_cases(n, seed):
     return cases
 
 
-@pytest.mark.parametrize("i,B,R,L,H,mode", _random_cases(28, 20261125))
+def _random_big_cases(n, seed):
+    # grids of several hundred workgroups and more: the eight-wave kernel in all its variants
+    import random
+
+    rng = random.Random(seed)
+    cases = []
+    for i in range(n):
+        H = rng.choice([16, 32, 64, 64, 128, 128])
+        L = rng.choice([rng.randint(520, 1100), rng.randint(1101, 2600), 8 * rng.randint(70, 300)])
+        B = rng.choice([1, 2, 4])
+        R = max(1, min(rng.choice([96, 200, 320, 512]) // B, 36_000_000 // (B * L * H)))
+        cases.append((100 + i, B, R, L, H, ["plain", "causal", "mask"][i % 3]))
+    return cases
+
+
+@pytest.mark.parametrize("i,B,R,L,H,mode", _random_cases(28, 20261125) + _random_big_cases(18, 20261126))
 def test_seeded_random_shapes(gpu, i, B, R, L, H, mode):
     # shapes drawn once from a fixed seed: odd lengths, every head_dim, grids from one workgroup to
     # several rounds of the chip, all three modes
