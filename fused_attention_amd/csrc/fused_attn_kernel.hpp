@@ -192,14 +192,10 @@ struct TileLoader {
 // Largest partial row sum (16 terms) the fast path of the online softmax accepts.
 constexpr float kTrip = 16384.f;
 
-// Eight-wave kernel: bias (log2 units) of the reference the exponentials are taken against, and what
-// its fast path accepts: with 64-row waves the largest sum of a query's 32 probabilities of one
-// sub-tile, with 32-row waves no packed pair of 16-bit floats (fp16 or bf16: 2.0 is 0x4000 in both)
-// with the "2.0 or more" bit set.
+// Eight-wave kernel: bias (log2 units) of the reference the exponentials are taken against, and the
+// largest sum of a query's 32 probabilities of one sub-tile that its fast path accepts.
 constexpr float kBias = 6.0f;
 constexpr float kTripSum = 32768.f;
-constexpr uint32_t kTripBits = 0x40004000u;
-__device__ __forceinline__ bool trips(uint32_t orv) { return (orv & kTripBits) != 0u; }
 
 // O^T[.][nb] *= alpha, in place.  Written as one instruction per register with the register tied
 // as input and output, so that the rarely taken rescale does not make the compiler keep a second
