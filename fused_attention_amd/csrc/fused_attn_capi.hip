@@ -23,12 +23,15 @@ struct Shape {
 };
 
 // Three shapes, picked by how the problem's workgroups fill the 256 compute units:
-//   {8, n}  eight waves of 64 (head_dim <= 64) or 32 (head_dim 128) query rows share one K/V
-//           stream, run by the ping-pong kernel; one such workgroup is resident per compute unit;
-//   {4, 2}  four 64-row waves, 256 queries per workgroup, two resident per compute unit;
+//   {8, 2}  eight 64-row waves share one K/V stream, run by the ping-pong kernel, 512 queries per
+//           workgroup, one resident per compute unit (head_dim <= 64 only: with head_dim 128 a
+//           64-row wave would need the whole register file of a SIMD);
+//   {8, 1}  the same kernel with 32-row waves, 256 queries per workgroup: the only ping-pong
+//           shape of head_dim 128 (one resident per compute unit); with head_dim <= 64 two are
+//           resident per compute unit and it serves the grids that {8, 2} fills badly (without
+//           mask only: the causal and the additive-mask variants do not fit 128 registers);
 //   {4, 1}  four 32-row waves, 128 queries per workgroup, three (head_dim <= 64) or two
 //           (head_dim 128) resident per compute unit: more, smaller workgroups for small problems.
-// head_dim 128 with 64-row waves needs the whole register file of a SIMD for one wave.
 int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // How well a shape uses the chip, in 1/1024: the share of the (rounds x slots) grid of resident
@@ -61,10 +64,11 @@ Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask, bool
     const bool pingpong = wgs8 >= 2 * kNumCu ? usage8 >= 614 : usage8 >= (wgs8 <= kNumCu ? 614 : 717);
     if (H > 64) return pingpong ? Shape{8, 1} : Shape{4, 1};
     if (pingpong) return {8, 2};
-    if (has_mask) return {4, 1};
-    // everything resident at once: the smallest workgroups give the most parallelism
-    if (heads * ceil_div(L, 128) <= 3 * kNumCu) return {4, 1};
-    return usage(heads, L, 256, 2 * kNumCu) > usage(heads, L, 128, 3 * kNumCu) ? Shape{4, 2} : Shape{4, 1};
+    // 256-query ping-pong workgroups, two per compute unit: per compute unit they run at 0.93 of
+    // the 512-query ones and 1.1 to 1.25 times as fast as the four-wave kernel, but they need 160
+    // or more workgroups to beat the latter's finer grain (sweep of 22 mid-size shapes on MI355X).
+    if (has_mask || causal) return {4, 1};
+    return heads * ceil_div(L, 256) >= 160 ? Shape{8, 1} : Shape{4, 1};
 }
 
 // Dynamic LDS above 64 KiB has to be opted into per kernel function and per device: done on the
@@ -116,14 +120,18 @@ hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) 
     if (sh.waves == 8) {
         if constexpr (H > 64)
             return launch_pingpong<H, 8, 1, 2, MODE, BF>(p, stream);
-        else
+        else if (sh.nqb == 2)
             return launch_pingpong<H, 8, 2, 2, MODE, BF>(p, stream);
+        else if constexpr (MODE == fa::kPlain)
+            return launch_pingpong<H, 8, 1, 4, MODE, BF>(p, stream);
+        else
+            return hipErrorInvalidValue;     // pick_shape never asks for this
     }
-    // four waves: 64-row waves where the registers allow it
+    // four 32-row waves; three per SIMD where the registers allow it
     if constexpr (H > 64 || MODE == fa::kAdditive)
         return launch<H, 4, 1, 2, MODE, BF>(p, stream);
     else
-        return sh.nqb == 2 ? launch<H, 4, 2, 2, MODE, BF>(p, stream) : launch<H, 4, 1, 3, MODE, BF>(p, stream);
+        return launch<H, 4, 1, 3, MODE, BF>(p, stream);
 }
 
 template <int MODE, bool BF>

@@ -416,8 +416,11 @@ def _check_pairs(got, q, k, v, H, pairs, mask=None):
 
 @pytest.mark.parametrize("B,R,L,H", [
     (1, 20, 4096, 64),      # eight-wave workgroups filling part of one round of the chip
-    (1, 40, 4096, 64),      # a poorly filled second round: four-wave workgroups instead
-    (1, 500, 256, 64),      # short sequences, 64-row waves
+    (1, 40, 4096, 64),      # a poorly filled second round: eight 32-row waves, two workgroups per CU
+    (1, 500, 256, 64),      # ... on short sequences
+    (2, 8, 3073, 64),       # ... with ragged tiles, less than one workgroup per CU
+    (1, 40, 2100, 32), (3, 20, 1111, 16),   # ... at the smaller head dims
+    (1, 32, 1024, 64),      # too few of those: four-wave workgroups
     (4, 16, 2112, 64),      # many workgroups, ragged last key tile and last query tile
     (1, 20, 2048, 128),     # head_dim 128, eight-wave workgroups in a part-filled round
     (1, 40, 2048, 128),     # head_dim 128, four-wave workgroups
@@ -536,6 +539,7 @@ BF16_TOL = 2e-2   # bf16 keeps 8 significant bits: the output rounding alone is 
     (4, 16, 2048, 64, False), (4, 16, 2048, 64, True),       # eight-wave kernel
     (2, 64, 1024, 128, False), (2, 64, 1024, 128, True),
     (2, 8, 1000, 64, False),
+    (2, 8, 3073, 64, False),                                  # eight 32-row waves, two workgroups per CU
 ])
 def test_bf16_inputs(gpu, B, R, L, H, causal):
     q, k, v = (_rand((B, L, R * H), 4200 + L + i).to(torch.bfloat16) for i in range(3))
