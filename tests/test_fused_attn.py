@@ -420,6 +420,7 @@ def _check_pairs(got, q, k, v, H, pairs, mask=None):
     (1, 500, 256, 64),      # ... on short sequences
     (2, 8, 3073, 64),       # ... with ragged tiles, less than one workgroup per CU
     (1, 40, 2100, 32), (3, 20, 1111, 16),   # ... at the smaller head dims
+    (1, 400, 40, 64), (2, 200, 7, 32),      # ... with sequences far shorter than a workgroup's 256 rows
     (1, 32, 1024, 64),      # too few of those: four-wave workgroups
     (4, 16, 2112, 64),      # many workgroups, ragged last key tile and last query tile
     (1, 20, 2048, 128),     # head_dim 128, eight-wave workgroups in a part-filled round
