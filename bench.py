@@ -26,7 +26,7 @@ PEAK_TFLOPS_FP16 = 2500.0   # MI355X dense fp16 MFMA, published
 # in separate --pmc runs of this script, each scaled by what the same counter reads for the 1 GiB
 # calibration copy below: 2.000 for fetch, 1.000 for write).  Summaries:
 # profiles/fwd_kernel_pingpong_c3.md and profiles/fwd_kernel_pingpong_c4.md.
-MEASURED_TRAFFIC_BYTES = {"c3": 134.4e6, "c4": 806.4e6}
+MEASURED_TRAFFIC_BYTES = {"c3": 134.4e6, "c4": 808.2e6}
 
 
 def cpu_baseline(w, q, k, v, gpu_out, budget_s):
