@@ -12,7 +12,8 @@
 //                        plain, causal and additive mask (mask rows 16-byte aligned)
 // Work decomposition
 //   workgroup  = NW wave64s, each wave owns 32 NQB query rows (NQB = 1 or 2 blocks of 32)
-//   K/V        = streamed in 64-key tiles, global -> registers -> LDS ring (2 or 3 slots)
+//   K/V        = streamed in 64-key tiles through an LDS ring: global -> registers -> LDS, two slots
+//                (fwd_kernel), or direct-to-LDS loads, three slots (fwd_kernel_pingpong)
 //   per 32 keys: S^T = K_sub * Q^T        v_mfma_f32_32x32x16_{f16,bf16}, Q held in registers
 //                online softmax on S^T     f32, state (m, l) per lane
 //                O^T += V_sub^T * P^T      same MFMA, V^T fetched with ds_read_b64_tr_b16
@@ -22,7 +23,7 @@
 // A softmax row therefore lives in one lane pair, so row max / row sum need 15 in-lane
 // ops and a single v_permlane32_swap.  The packed 16-bit P^T registers are, as they stand,
 // a valid B operand of the second product provided the A operand (V^T) enumerates keys
-// in the same order, which the transpose-read from a row-major V tile provides.
+// in the same order, which the transpose-read from the V tile provides.
 //
 // MFMA operand maps used below (g = lane / 32, ln = lane % 32):
 //   A (32 x 16): lane holds row ln,   k = 8 g + i          (i = 0..7)
