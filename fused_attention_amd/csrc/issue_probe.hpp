@@ -219,5 +219,171 @@ inline int issue_probe() {
     (void)hipFree(data);
     return 0;
 }
+// Phase probe, run as `fa_test phase-probe`: the compute of the eight-wave attention kernel at
+// head_dim 64 with everything else taken away (no LDS, no global memory in the loop).  On every
+// compute unit two groups of four waves alternate, with a workgroup barrier between phases, between
+// the 20 matrix instructions of a 32-key x 64-query sub-tile (4 row-sum MFMAs, 8 for QK^T, 8 for PV,
+// with the kernel's dependency pattern) and its 32 fma + 32 exp + 16 pack.  Reported per phase:
+// wall time, the clocks each kind of phase takes from barrier to barrier, and the shader clock.
+typedef float f4v __attribute__((ext_vector_type(4)));
+typedef unsigned u4v __attribute__((ext_vector_type(4)));
+
+template <int VWORK, int STAMPS>
+__global__ __launch_bounds__(512) void phase_kernel(float* out, long long* clk, const h8* data, int iters, float c,
+                                                    float mc) {
+    const int wave = threadIdx.x / 64;
+    const int grp = (wave >> 2) & 1;
+    h8 a[8], q[8];
+    for (int i = 0; i < 8; i++) {
+        a[i] = data[threadIdx.x + i * 512];
+        q[i] = data[threadIdx.x + (i + 8) * 512];
+    }
+    f16v s[2], o[4];
+    f4v l[2];
+    unsigned pk[2][8];
+    for (int n = 0; n < 2; n++) {
+        for (int r = 0; r < 16; r++) s[n][r] = 0.01f * r;
+        for (int i = 0; i < 8; i++) pk[n][i] = 0x2c002c00u;
+        l[n] = f4v{0.f, 0.f, 0.f, 0.f};
+    }
+    for (int n = 0; n < 4; n++)
+        for (int r = 0; r < 16; r++) o[n][r] = 0.f;
+    unsigned long long t0 = 0, t1 = 0, t2 = 0, r0 = 0, first = 0, mwork = 0, vwork = 0;
+    for (int it = 0; it < iters; it++) {
+        if (STAMPS) {
+            asm volatile("s_memtime %0" : "=s"(t0));
+            if (it == iters - 64) asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r0)::"memory");
+        }
+        if (grp == (it & 1)) {
+            __builtin_amdgcn_s_setprio(3);
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int n = 0; n < 2; n++) {
+                    const u4v w = {pk[n][4 * t], pk[n][4 * t + 1], pk[n][4 * t + 2], pk[n][4 * t + 3]};
+                    l[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[7], __builtin_bit_cast(h8, w), l[n], 0, 0, 0);
+                }
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for (int n = 0; n < 2; n++) {
+                    f16v z;
+                    for (int r = 0; r < 16; r++) z[r] = 0.f;
+                    s[n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[kk], q[kk * 2 + n], kk == 0 ? z : s[n], 0, 0, 0);
+                }
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int db = 0; db < 2; db++)
+#pragma unroll
+                    for (int n = 0; n < 2; n++) {
+                        const u4v w = {pk[n][4 * t], pk[n][4 * t + 1], pk[n][4 * t + 2], pk[n][4 * t + 3]};
+                        o[db * 2 + n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[4 + t * 2 + db], __builtin_bit_cast(h8, w),
+                                                                               o[db * 2 + n], 0, 0, 0);
+                    }
+            __builtin_amdgcn_s_setprio(0);
+        } else if (VWORK) {
+#pragma unroll
+            for (int n = 0; n < 2; n++)
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[n][r], c, mc));
+                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[n][r + 1], c, mc));
+                    pk[n][r >> 1] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pkrtz(p0, p1));
+                }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (STAMPS)
+            asm volatile("s_memtime %0\n\ts_barrier\n\ts_memtime %1\n\ts_waitcnt lgkmcnt(0)" : "=s"(t1), "=s"(t2)::"memory");
+        else
+            __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        // the last 64 phases, kept in scalar registers: work of this wave per kind of phase, and the
+        // release of the barrier that ends the phase
+        if (it == iters - 65) first = t2;
+        if (it >= iters - 64) {
+            if (grp == (it & 1)) mwork += t1 - t0; else vwork += t1 - t0;
+        }
+    }
+    if (STAMPS && blockIdx.x == 0 && threadIdx.x % 64 == 0) {
+        unsigned long long r1;
+        asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r1)::"memory");
+        long long* p = clk + wave * 4;
+        p[0] = (long long)mwork;
+        p[1] = (long long)vwork;
+        p[2] = (long long)(t2 - first);
+        p[3] = (long long)(r1 - r0);
+    }
+    float acc = 0.f;
+    for (int n = 0; n < 2; n++) {
+        for (int r = 0; r < 16; r++) acc += s[n][r];
+        acc += l[n][0];
+    }
+    for (int n = 0; n < 4; n++)
+        for (int r = 0; r < 16; r++) acc += o[n][r];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = acc;
+}
+
+template <int VWORK, int STAMPS>
+int run_phase(const char* name, int blocks, float* out, long long* clk, const h8* data) {
+    const int iters = 20000;
+    hipEvent_t e0, e1;
+    PROBE_OK(hipEventCreate(&e0));
+    PROBE_OK(hipEventCreate(&e1));
+    hipLaunchKernelGGL((phase_kernel<VWORK, STAMPS>), dim3(blocks), dim3(512), 0, nullptr, out, clk, data, 2000, 0.18f, -1.0f);
+    PROBE_OK(hipEventRecord(e0, nullptr));
+    hipLaunchKernelGGL((phase_kernel<VWORK, STAMPS>), dim3(blocks), dim3(512), 0, nullptr, out, clk, data, iters, 0.18f, -1.0f);
+    PROBE_OK(hipEventRecord(e1, nullptr));
+    PROBE_OK(hipEventSynchronize(e1));
+    float ms = 0.f;
+    PROBE_OK(hipEventElapsedTime(&ms, e0, e1));
+    long long h[32];
+    PROBE_OK(hipMemcpy(h, clk, sizeof(h), hipMemcpyDeviceToHost));
+    // wave 0 of workgroup 0: 32 matrix and 32 vector phases among its last 64
+    const double phase_clk = (double)h[2] / 64.0;
+    const double ghz = (double)h[2] / ((double)h[3] * 10.0);
+    if (STAMPS)
+        std::printf("  %-34s %6.1f ns per phase | with stamps: %5.0f clocks per phase, matrix work %4.0f, vector work %4.0f, %.2f GHz\n",
+                    name, ms * 1e6 / iters, phase_clk, (double)h[0] / 32.0, (double)h[1] / 32.0, ghz);
+    else
+        std::printf("  %-34s %6.1f ns per phase\n", name, ms * 1e6 / iters);
+    return 0;
+}
+
+inline int phase_probe() {
+    hipDeviceProp_t prop;
+    PROBE_OK(hipGetDeviceProperties(&prop, 0));
+    const int blocks = prop.multiProcessorCount;
+    float* out;
+    long long* clk;
+    h8* data;
+    PROBE_OK(hipMalloc(&out, (size_t)blocks * 512 * 4));
+    PROBE_OK(hipMalloc(&clk, 32 * sizeof(long long)));
+    PROBE_OK(hipMalloc(&data, 16 * 512 * sizeof(h8)));
+    _Float16* host = new _Float16[16 * 512 * 8];
+    unsigned st = 1u;
+    for (int i = 0; i < 16 * 512 * 8; i++) {     // sum of 12 uniforms - 6: close to N(0,1)
+        float u = 0.f;
+        for (int k = 0; k < 12; k++) {
+            st = st * 1664525u + 1013904223u;
+            u += (float)(st >> 8) / 16777216.0f;
+        }
+        host[i] = (_Float16)(u - 6.0f);
+    }
+    PROBE_OK(hipMemcpy(data, host, 16 * 512 * sizeof(h8), hipMemcpyHostToDevice));
+    delete[] host;
+    std::printf("phase-probe: two groups of four waves per compute unit alternate between the matrix and the vector work of one\n"
+                "32-key x 64-query sub-tile at head_dim 64 (N(0,1) operands, no memory traffic), %d compute units\n", blocks);
+    for (int rep = 0; rep < 2; rep++) {
+        if (run_phase<0, 0>("matrix phases only", blocks, out, clk, data)) return 2;
+        if (run_phase<1, 0>("matrix and vector phases", blocks, out, clk, data)) return 2;
+        if (run_phase<0, 1>("matrix phases only", blocks, out, clk, data)) return 2;
+        if (run_phase<1, 1>("matrix and vector phases", blocks, out, clk, data)) return 2;
+    }
+    (void)hipFree(out);
+    (void)hipFree(clk);
+    (void)hipFree(data);
+    return 0;
+}
 
 }  // namespace probe
