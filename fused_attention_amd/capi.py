@@ -11,7 +11,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libfused_attn_gfx950.so")
 
 # every symbol include/fused_attn.h declares
-EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_query", "fa_strerror", "fa_fwd_timed")
+EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_strided", "fa_fwd_query", "fa_strerror", "fa_fwd_timed")
 FLAG_CAUSAL = 1
 FLAG_BF16 = 2
 
@@ -43,6 +43,9 @@ def load_library():
     lib.fa_fwd_ex.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, f32,
                               ctypes.c_int, vp]
     lib.fa_fwd_ex.restype = ctypes.c_int
+    lib.fa_fwd_strided.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, i64, i64,
+                                   f32, ctypes.c_int, vp]
+    lib.fa_fwd_strided.restype = ctypes.c_int
     lib.fa_fwd_timed.argtypes = fwd_args + [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
     lib.fa_fwd_timed.restype = ctypes.c_int
     lib.fa_fwd_query.argtypes = [i64]
@@ -80,6 +83,15 @@ def _layout(q, head_dim, layout):
     raise ValueError("layout must be 'blf' or 'bhld'")
 
 
+def _strides(t, head_dim, layout, name):
+    """(stride_b, stride_h, stride_l) in elements of a tensor or view whose last dimension is dense."""
+    if t.stride(-1) != 1:
+        raise ValueError("%s: the last dimension must be contiguous" % name)
+    if layout == "blf":
+        return t.stride(0), head_dim, t.stride(1)
+    return t.stride(0), t.stride(1), t.stride(2)
+
+
 def _current_stream(q):
     import torch
 
@@ -88,10 +100,12 @@ def _current_stream(q):
 
 def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None, causal=False,
             return_lse=False):
-    """Runs fa_fwd_ex on torch GPU tensors (fp16 or bf16, contiguous) on torch's current stream.
+    """Runs fa_fwd_strided on torch GPU tensors (fp16 or bf16) on torch's current stream.
 
     layout 'blf' takes [B, L, R*head_dim] tensors, 'bhld' takes [B, R, L, head_dim] tensors.
-    causal=True restricts query i to keys j <= i.  q, k, v (and out, mask when given) must share
+    q, k and v may be views (slices of one packed projection output, say) as long as their last
+    dimension is dense and the three have the same strides; `out` may be a view of its own.  The
+    mask is contiguous [B, L, L].  causal=True restricts query i to keys j <= i.  q, k, v (and out, mask when given) must share
     one dtype; bfloat16 tensors set FA_FLAG_BF16.  Returns `out` (allocated like q when not
     given), or (out, lse) with lse a float32 [B, R, L] tensor when return_lse is set.
     """
@@ -103,17 +117,27 @@ def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None, ca
         if t is not None and t.dtype != q.dtype:
             raise TypeError("%s must have the dtype of q (%s), got %s" % (name, q.dtype, t.dtype))
     flags = (FLAG_CAUSAL if causal else 0) | (FLAG_BF16 if q.dtype == torch.bfloat16 else 0)
-    B, R, L, sb, sh, sl = _layout(q, head_dim, layout)
+    B, R, L = _layout(q, head_dim, layout)[:3]
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("q, k, v must have one shape")
+    sb, sh, sl = _strides(q, head_dim, layout, "q")
+    if _strides(k, head_dim, layout, "k") != (sb, sh, sl) or _strides(v, head_dim, layout, "v") != (sb, sh, sl):
+        raise ValueError("q, k, v must have the same strides")
+    if mask is not None and not mask.is_contiguous():
+        raise ValueError("mask must be contiguous")
     if out is None:
-        out = torch.empty_like(q)
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    elif out.shape != q.shape:
+        raise ValueError("out must have the shape of q")
+    ob, oh, ol = _strides(out, head_dim, layout, "out")
     if scale is None:
         scale = 1.0 / math.sqrt(head_dim)
     lse = torch.empty((B, R, L), dtype=torch.float32, device=q.device) if return_lse else None
     with torch.cuda.device(q.device):
-        status = load_library().fa_fwd_ex(
+        status = load_library().fa_fwd_strided(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr() if mask is not None else None,
             out.data_ptr(), lse.data_ptr() if lse is not None else None, B, R, L, head_dim, sb, sh, sl,
-            scale, flags, _current_stream(q) or None)
+            ob, oh, ol, scale, flags, _current_stream(q) or None)
     _check(status)
     return (out, lse) if return_lse else out
 

@@ -152,14 +152,27 @@ hipError_t dispatch(int64_t H, Shape sh, const fa::FwdParams& p, hipStream_t str
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
+struct Strides {
+    int64_t b, h, l;
+};
+
+bool strides_ok(const Strides& s, int64_t H) {
+    return s.l >= H && s.h >= 0 && s.b >= 0 && (s.l % 8) == 0 && (s.h % 8) == 0 && (s.b % 8) == 0;
+}
+
+bool extent_ok(const Strides& s, int64_t B, int64_t R, int64_t L) {
+    constexpr int64_t kMaxElems = (int64_t)1 << 62;
+    return !(L > kMaxElems / s.l || (s.h > 0 && R > kMaxElems / s.h) || (s.b > 0 && B > kMaxElems / s.b));
+}
+
 int validate(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,
-             int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h, int64_t stride_l,
+             int64_t R, int64_t L, int64_t H, const Strides& in, const Strides& os,
              fa::FwdParams* p, float scale, Shape* shape, bool causal, void* lse) {
+    const int64_t stride_b = in.b, stride_h = in.h, stride_l = in.l;
     if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return FA_ERR_NULL_POINTER;
     if (!fa_fwd_query(H)) return FA_ERR_BAD_HEAD_DIM;
     if (B < 1 || R < 1 || L < 1) return FA_ERR_BAD_SHAPE;
-    if (stride_l < H || stride_h < 0 || stride_b < 0) return FA_ERR_BAD_STRIDE;
-    if ((stride_l % 8) != 0 || (stride_h % 8) != 0 || (stride_b % 8) != 0) return FA_ERR_BAD_STRIDE;
+    if (!strides_ok(in, H) || !strides_ok(os, H)) return FA_ERR_BAD_STRIDE;
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return FA_ERR_MISALIGNED;
     if (mask != nullptr && (reinterpret_cast<uintptr_t>(mask) & 1u) != 0) return FA_ERR_MISALIGNED;
     constexpr int64_t kMaxInt = 0x7fffffff;
@@ -173,10 +186,7 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     if (causal && shape->waves == 8) n_qtiles = (n_qtiles + 1) / 2;   // pairs of query tiles
     const int64_t total = B * R * n_qtiles;
     if (total > kMaxInt - 8 || B * R > kMaxInt) return FA_ERR_TOO_LARGE;
-    constexpr int64_t kMaxElems = (int64_t)1 << 62;
-    if (L > kMaxElems / stride_l || (stride_h > 0 && R > kMaxElems / stride_h) ||
-        (stride_b > 0 && B > kMaxElems / stride_b))
-        return FA_ERR_TOO_LARGE;
+    if (!extent_ok(in, B, R, L) || !extent_ok(os, B, R, L)) return FA_ERR_TOO_LARGE;
 
     p->q = static_cast<const _Float16*>(q);
     p->k = static_cast<const _Float16*>(k);
@@ -187,6 +197,9 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     p->stride_b = stride_b;
     p->stride_h = stride_h;
     p->stride_l = stride_l;
+    p->ostride_b = os.b;
+    p->ostride_h = os.h;
+    p->ostride_l = os.l;
     p->B = (int)B;
     p->R = (int)R;
     p->L = (int)L;
@@ -220,9 +233,10 @@ const char* fa_strerror(int status) {
     return "fa_fwd: unknown status";
 }
 
-int fa_fwd_ex(const void* q, const void* k, const void* v, const void* mask, void* out, void* lse,
-              int64_t B, int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h,
-              int64_t stride_l, float scale, int flags, void* stream) {
+int fa_fwd_strided(const void* q, const void* k, const void* v, const void* mask, void* out, void* lse,
+                   int64_t B, int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h,
+                   int64_t stride_l, int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_l,
+                   float scale, int flags, void* stream) {
     if ((flags & ~(FA_FLAG_CAUSAL | FA_FLAG_BF16)) != 0) return FA_ERR_BAD_FLAGS;
     const bool causal = (flags & FA_FLAG_CAUSAL) != 0;
     const bool bf16 = (flags & FA_FLAG_BF16) != 0;
@@ -230,8 +244,8 @@ int fa_fwd_ex(const void* q, const void* k, const void* v, const void* mask, voi
     if (lse != nullptr && (reinterpret_cast<uintptr_t>(lse) & 3u) != 0) return FA_ERR_MISALIGNED;
     fa::FwdParams p;
     Shape shape{4, 2};
-    const int rc = validate(q, k, v, mask, out, B, R, L, H, stride_b, stride_h, stride_l, &p, scale,
-                            &shape, causal, lse);
+    const int rc = validate(q, k, v, mask, out, B, R, L, H, Strides{stride_b, stride_h, stride_l},
+                            Strides{out_stride_b, out_stride_h, out_stride_l}, &p, scale, &shape, causal, lse);
     if (rc != FA_OK) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e;
@@ -242,6 +256,13 @@ int fa_fwd_ex(const void* q, const void* k, const void* v, const void* mask, voi
     else
         e = dispatch<fa::kPlain>(H, shape, p, s, bf16);
     return static_cast<int>(e);
+}
+
+int fa_fwd_ex(const void* q, const void* k, const void* v, const void* mask, void* out, void* lse,
+              int64_t B, int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h,
+              int64_t stride_l, float scale, int flags, void* stream) {
+    return fa_fwd_strided(q, k, v, mask, out, lse, B, R, L, H, stride_b, stride_h, stride_l, stride_b, stride_h,
+                          stride_l, scale, flags, stream);
 }
 
 int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,

@@ -54,9 +54,12 @@ struct FwdParams {
     const _Float16* mask;  // additive [B, L, L] or nullptr
     _Float16* o;
     float* lse;            // optional [B, R, L] natural-log row sums of exp(scores), or nullptr
-    int64_t stride_b;      // elements between batches
-    int64_t stride_h;      // elements between heads
-    int64_t stride_l;      // elements between sequence positions
+    int64_t stride_b;      // q, k, v: elements between batches
+    int64_t stride_h;      // ... between heads
+    int64_t stride_l;      // ... between sequence positions
+    int64_t ostride_b;     // the same three for o
+    int64_t ostride_h;
+    int64_t ostride_l;
     int B, R, L;
     int n_qtiles;          // workgroups per (batch, head): ceil(L / queries per workgroup), or half of
                            // that (rounded up) when a causal workgroup takes a pair of query tiles

@@ -80,6 +80,22 @@ int fa_fwd_ex(const void* q, const void* k, const void* v, const void* mask, voi
               float scale, int flags, void* stream);
 
 /*
+ * fa_fwd_ex with strides of its own for `out`: q, k and v share (stride_b, stride_h, stride_l),
+ * out is addressed with (out_stride_b, out_stride_h, out_stride_l), under the same rules
+ * (multiples of 8 elements, last dimension contiguous; the 2^24 limit applies to stride_l only).
+ * This is what lets q, k and v be three views into one packed projection output (say
+ * [B, L, 3, R, H], the layout a fused QKV projection writes: reference README.md:137 lists that
+ * front end as not done) while out is an ordinary contiguous tensor, with no copy on either side.
+ * The reference has no counterpart: its launcher takes contiguous [B, L, R*H] tensors only
+ * (reference src/fused_attn_extention.cu:34-44).
+ */
+int fa_fwd_strided(const void* q, const void* k, const void* v, const void* mask, void* out, void* lse,
+                   int64_t B, int64_t R, int64_t L, int64_t H,
+                   int64_t stride_b, int64_t stride_h, int64_t stride_l,
+                   int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_l,
+                   float scale, int flags, void* stream);
+
+/*
  * 1 if fa_fwd accepts this head_dim, else 0.  Counterpart of the compile-time
  * (head_dim, chunk_size) dispatch table (reference src/fused_attn_extention.cu:72-111).
  */

@@ -55,6 +55,17 @@ def test_status_codes_for_rejected_arguments():
     lib = capi.load_library()
     assert lib.fa_fwd_ex(ok_ptr, ok_ptr, ok_ptr, None, ok_ptr, None, B, R, L, H, L * R * H, H, R * H, 0.125, 4, None) == -7
     assert lib.fa_fwd_ex(ok_ptr, ok_ptr, ok_ptr, ok_ptr, ok_ptr, None, B, R, L, H, L * R * H, H, R * H, 0.125, 1, None) == -7
+    def strided(in_strides, out_strides, flags=0):
+        return lib.fa_fwd_strided(ok_ptr, ok_ptr, ok_ptr, None, ok_ptr, None, B, R, L, H, *in_strides, *out_strides,
+                                  0.125, flags, None)
+
+    packed = (L * 3 * R * H, H, 3 * R * H)       # q, k, v as slices of [B, L, 3, R, H]
+    dense = (L * R * H, H, R * H)
+    assert strided(packed, (L * R * H, H, H - 8)) == -4       # output rows would overlap
+    assert strided(packed, (L * R * H, H + 4, R * H)) == -4   # output heads not 16-byte aligned
+    assert strided((L * R * H, H, R * H + 2), dense) == -4
+    assert strided(packed, (2 ** 62 + 8, H, R * H)) == -6         # output extent beyond the index range
+    assert strided(packed, dense, flags=8) == -7
     for code in (-1, -2, -3, -4, -5, -6, -7):
         assert "fa_fwd" in capi.strerror(code)
     assert capi.strerror(0) == "success"

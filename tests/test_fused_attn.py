@@ -157,6 +157,50 @@ def test_native_bhld_layout_matches_packed_layout(gpu):
     assert torch.equal(native.transpose(1, 2).reshape(B, L, R * H), packed)
 
 
+@pytest.mark.parametrize("B,R,L,H,mode", [
+    (2, 3, 200, 64, "plain"), (1, 2, 333, 128, "plain"), (2, 4, 130, 16, "plain"), (3, 2, 257, 32, "causal"),
+    (1, 2, 200, 64, "mask"), (4, 16, 2048, 64, "plain"), (1, 32, 2048, 128, "causal"), (2, 80, 512, 64, "plain"),
+])
+def test_views_into_a_packed_qkv_tensor(gpu, B, R, L, H, mode):
+    """q, k, v as slices of one [B, L, 3, R*H] projection output and a dense output of its own
+    strides: bitwise the result of the same call on contiguous copies, and the packed tensor's
+    other bytes (and the padding around a strided output) stay untouched."""
+    F = R * H
+    qkv = _rand((B, L, 3, F), 77 + L).to(gpu)
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    assert not q.is_contiguous()
+    mask = None
+    if mode == "mask":
+        mask = (_rand((B, L, L), 5) * 2).to(gpu)
+    kw = dict(mask=mask, causal=(mode == "causal"), return_lse=True)
+    want, want_lse = capi.forward(q.contiguous(), k.contiguous(), v.contiguous(), H, **kw)
+    before = qkv.clone()
+    got, got_lse = capi.forward(q, k, v, H, **kw)
+    assert got.is_contiguous() and torch.equal(got, want) and torch.equal(got_lse, want_lse)
+    assert torch.equal(qkv, before)
+    # the output as a view as well: every second row slot of a padded buffer
+    pad = torch.full((B, L, 2, F + 8), 7.0, dtype=torch.float16, device=gpu)
+    view = pad[:, :, 1, 8:]
+    capi.forward(q, k, v, H, out=view, mask=mask, causal=(mode == "causal"))
+    assert torch.equal(view, want)
+    assert (pad[:, :, 0] == 7.0).all() and (pad[:, :, 1, :8] == 7.0).all()
+    if L <= 400:
+        omask = causal_mask(B, L) if mode == "causal" else (mask.cpu() if mask is not None else None)
+        assert _max_err(got, attention(*(t.contiguous().cpu() for t in (q, k, v)), H, mask=omask)) <= TOL
+
+
+def test_views_in_the_bhld_layout_and_mismatched_strides(gpu):
+    B, R, L, H = 2, 3, 150, 64
+    big = _rand((3, B, R, L + 10, H), 9).to(gpu)          # [3][B, R, L+10, H]: rows beyond L are padding
+    q, k, v = (big[i, :, :, :L] for i in range(3))
+    want = capi.forward(q.contiguous(), k.contiguous(), v.contiguous(), H, layout="bhld")
+    assert torch.equal(capi.forward(q, k, v, H, layout="bhld"), want)
+    with pytest.raises(ValueError, match="same strides"):
+        capi.forward(q, k.contiguous(), v, H, layout="bhld")
+    with pytest.raises(ValueError, match="last dimension"):
+        capi.forward(q.transpose(2, 3).contiguous().transpose(2, 3), k, v, H, layout="bhld")
+
+
 def test_runs_on_the_current_stream_and_is_deterministic(gpu):
     import fused_attn
 
