@@ -225,6 +225,11 @@ inline int issue_probe() {
 // the 20 matrix instructions of a 32-key x 64-query sub-tile (4 row-sum MFMAs, 8 for QK^T, 8 for PV,
 // with the kernel's dependency pattern) and its 32 fma + 32 exp + 16 pack.  Reported per phase:
 // wall time, the clocks each kind of phase takes from barrier to barrier, and the shader clock.
+// VWORK selects the work: 0 matrix phases only, 1 the kernel's split, and three splits the kernel
+// does not use, timed for comparison: 2 the reference folded into QK^T as a fifth k-step (no fma
+// in the vector phase), 3 row sums by v_add_f32 (no row-sum MFMAs), 4 pairs of packed
+// probabilities added in fp16 first (half the row-sum MFMAs).
+typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 typedef float f4v __attribute__((ext_vector_type(4)));
 typedef unsigned u4v __attribute__((ext_vector_type(4)));
 
@@ -240,10 +245,11 @@ __global__ __launch_bounds__(512) void phase_kernel(float* out, long long* clk, 
     }
     f16v s[2], o[4];
     f4v l[2];
-    unsigned pk[2][8];
+    unsigned pk[2][8], ps[2][4];
     for (int n = 0; n < 2; n++) {
         for (int r = 0; r < 16; r++) s[n][r] = 0.01f * r;
         for (int i = 0; i < 8; i++) pk[n][i] = 0x2c002c00u;
+        for (int i = 0; i < 4; i++) ps[n][i] = 0x2c002c00u;
         l[n] = f4v{0.f, 0.f, 0.f, 0.f};
     }
     for (int n = 0; n < 4; n++)
@@ -257,19 +263,21 @@ __global__ __launch_bounds__(512) void phase_kernel(float* out, long long* clk, 
         if (grp == (it & 1)) {
             __builtin_amdgcn_s_setprio(3);
 #pragma unroll
-            for (int t = 0; t < 2; t++)
+            for (int t = 0; t < (VWORK == 3 ? 0 : VWORK == 4 ? 1 : 2); t++)
 #pragma unroll
                 for (int n = 0; n < 2; n++) {
-                    const u4v w = {pk[n][4 * t], pk[n][4 * t + 1], pk[n][4 * t + 2], pk[n][4 * t + 3]};
+                    const u4v w = VWORK == 4 ? u4v{ps[n][0], ps[n][1], ps[n][2], ps[n][3]}
+                                             : u4v{pk[n][4 * t], pk[n][4 * t + 1], pk[n][4 * t + 2], pk[n][4 * t + 3]};
                     l[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[7], __builtin_bit_cast(h8, w), l[n], 0, 0, 0);
                 }
 #pragma unroll
-            for (int kk = 0; kk < 4; kk++)
+            for (int kk = 0; kk < (VWORK == 2 ? 5 : 4); kk++)
 #pragma unroll
                 for (int n = 0; n < 2; n++) {
                     f16v z;
                     for (int r = 0; r < 16; r++) z[r] = 0.f;
-                    s[n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[kk], q[kk * 2 + n], kk == 0 ? z : s[n], 0, 0, 0);
+                    s[n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kk == 4 ? a[6] : a[kk], kk == 4 ? q[n] : q[kk * 2 + n],
+                                                                  kk == 0 ? z : s[n], 0, 0, 0);
                 }
 #pragma unroll
             for (int t = 0; t < 2; t++)
@@ -284,13 +292,24 @@ __global__ __launch_bounds__(512) void phase_kernel(float* out, long long* clk, 
             __builtin_amdgcn_s_setprio(0);
         } else if (VWORK) {
 #pragma unroll
-            for (int n = 0; n < 2; n++)
+            for (int n = 0; n < 2; n++) {
 #pragma unroll
                 for (int r = 0; r < 16; r += 2) {
-                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[n][r], c, mc));
-                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[n][r + 1], c, mc));
+                    const float p0 = __builtin_amdgcn_exp2f(VWORK == 2 ? s[n][r] : __builtin_fmaf(s[n][r], c, mc));
+                    const float p1 = __builtin_amdgcn_exp2f(VWORK == 2 ? s[n][r + 1] : __builtin_fmaf(s[n][r + 1], c, mc));
                     pk[n][r >> 1] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pkrtz(p0, p1));
+                    if (VWORK == 3) {
+                        l[n][r & 3] += p0;
+                        l[n][(r + 1) & 3] += p1;
+                    }
                 }
+                if (VWORK == 4) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        ps[n][i] = __builtin_bit_cast(unsigned, __builtin_bit_cast(h2v, pk[n][i]) +
+                                                                    __builtin_bit_cast(h2v, pk[n][i + 4]));
+                }
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         if (STAMPS)
@@ -379,6 +398,9 @@ inline int phase_probe() {
         if (run_phase<1, 0>("matrix and vector phases", blocks, out, clk, data)) return 2;
         if (run_phase<0, 1>("matrix phases only", blocks, out, clk, data)) return 2;
         if (run_phase<1, 1>("matrix and vector phases", blocks, out, clk, data)) return 2;
+        if (run_phase<2, 0>("reference as a fifth k-step, no fma", blocks, out, clk, data)) return 2;
+        if (run_phase<3, 0>("row sums by v_add_f32", blocks, out, clk, data)) return 2;
+        if (run_phase<4, 0>("half the row-sum mfma, pk_add_f16", blocks, out, clk, data)) return 2;
     }
     (void)hipFree(out);
     (void)hipFree(clk);
