@@ -440,6 +440,33 @@ def test_lse_of_the_pingpong_kernel(gpu):
     assert _max_err(out, want) <= 1e-3
 
 
+@pytest.mark.parametrize("R,H,causal", [(48, 64, False), (24, 128, False), (24, 64, True)])
+def test_very_long_ragged_sequence(gpu, R, H, causal):
+    """L = 65537: 1025 key tiles with a single key in the last one, 129 (257) query tiles with a
+    single query in the last one.  One head against the oracle on sampled query rows (the full
+    L x L scores of one head would be 17 GB), every head against closed forms."""
+    B, L = 1, 65537
+    q, k, v = (_rand((B, L, R * H), 6500 + H + i) for i in range(3))
+    got, lse = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, causal=causal, return_lse=True)
+    got, lse = got.float().cpu(), lse.cpu()
+    assert torch.isfinite(got).all() and torch.isfinite(lse).all()
+    rows = torch.tensor([0, 1, 31, 32, 255, 256, 511, 512, 4095, 32768, 65023, 65024, 65535, 65536])
+    h = R - 1
+    sl = slice(h * H, (h + 1) * H)
+    scores = (q[0, rows, sl].float() @ k[0, :, sl].float().T) / math.sqrt(H)
+    if causal:
+        scores = scores.masked_fill(torch.arange(L)[None, :] > rows[:, None], float("-inf"))
+    want = torch.softmax(scores, dim=-1) @ v[0, :, sl].float()
+    assert (got[0, rows, sl] - want).abs().max().item() <= TOL
+    assert (lse[0, h, rows] - torch.logsumexp(scores, dim=-1)).abs().max().item() <= 1e-3 * math.log(L)
+    # outputs are convex combinations of the value rows
+    assert (got.abs().amax(dim=1) <= v.float().abs().amax(dim=1) + 1e-3).all()
+    if not causal:
+        zero = capi.forward(torch.zeros_like(q).to(gpu), k.to(gpu), v.to(gpu), H).float().cpu()
+        mean = v.float().mean(dim=1, keepdim=True)
+        assert (zero - mean).abs().max().item() <= 1e-3
+
+
 # ---- every launch shape, plain and masked -------------------------------------------------------------
 
 def _check_pairs_tol(got, q, k, v, H, pairs, mask, tol):
