@@ -229,6 +229,9 @@ inline int issue_probe() {
 // does not use, timed for comparison: 2 the reference folded into QK^T as a fifth k-step (no fma
 // in the vector phase), 3 row sums by v_add_f32 (no row-sum MFMAs), 4 pairs of packed
 // probabilities added in fp16 first (half the row-sum MFMAs).
+// STAMPS selects the clock readings: 0 none, 1 around every barrier (work per kind of phase; the
+// readings themselves add about 250 clocks to a phase), 2 two readings around the last 1024
+// phases (clocks per phase and shader clock of the undisturbed loop).
 typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 typedef float f4v __attribute__((ext_vector_type(4)));
 typedef unsigned u4v __attribute__((ext_vector_type(4)));
@@ -256,7 +259,11 @@ __global__ __launch_bounds__(512) void phase_kernel(float* out, long long* clk, 
         for (int r = 0; r < 16; r++) o[n][r] = 0.f;
     unsigned long long t0 = 0, t1 = 0, t2 = 0, r0 = 0, first = 0, mwork = 0, vwork = 0;
     for (int it = 0; it < iters; it++) {
-        if (STAMPS) {
+        if (STAMPS == 2) {      // two stamps for the whole run: the last 1024 phases
+            if (it == iters - 1024)
+                asm volatile("s_memtime %0\n\ts_memrealtime %1\n\ts_waitcnt lgkmcnt(0)" : "=s"(first), "=s"(r0)::"memory");
+        }
+        if (STAMPS == 1) {
             asm volatile("s_memtime %0" : "=s"(t0));
             if (it == iters - 64) asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r0)::"memory");
         }
@@ -312,20 +319,21 @@ __global__ __launch_bounds__(512) void phase_kernel(float* out, long long* clk, 
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (STAMPS)
+        if (STAMPS == 1)
             asm volatile("s_memtime %0\n\ts_barrier\n\ts_memtime %1\n\ts_waitcnt lgkmcnt(0)" : "=s"(t1), "=s"(t2)::"memory");
         else
             __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         // the last 64 phases, kept in scalar registers: work of this wave per kind of phase, and the
         // release of the barrier that ends the phase
-        if (it == iters - 65) first = t2;
-        if (it >= iters - 64) {
+        if (STAMPS == 1 && it == iters - 65) first = t2;
+        if (STAMPS == 1 && it >= iters - 64) {
             if (grp == (it & 1)) mwork += t1 - t0; else vwork += t1 - t0;
         }
     }
     if (STAMPS && blockIdx.x == 0 && threadIdx.x % 64 == 0) {
         unsigned long long r1;
+        if (STAMPS == 2) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t2)::"memory");
         asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r1)::"memory");
         long long* p = clk + wave * 4;
         p[0] = (long long)mwork;
@@ -359,9 +367,11 @@ int run_phase(const char* name, int blocks, float* out, long long* clk, const h8
     long long h[32];
     PROBE_OK(hipMemcpy(h, clk, sizeof(h), hipMemcpyDeviceToHost));
     // wave 0 of workgroup 0: 32 matrix and 32 vector phases among its last 64
-    const double phase_clk = (double)h[2] / 64.0;
+    const double phase_clk = (double)h[2] / (STAMPS == 2 ? 1024.0 : 64.0);
     const double ghz = (double)h[2] / ((double)h[3] * 10.0);
-    if (STAMPS)
+    if (STAMPS == 2)
+        std::printf("  %-34s %6.1f ns per phase | %5.0f clocks per phase at %.2f GHz\n", name, ms * 1e6 / iters, phase_clk, ghz);
+    else if (STAMPS)
         std::printf("  %-34s %6.1f ns per phase | with stamps: %5.0f clocks per phase, matrix work %4.0f, vector work %4.0f, %.2f GHz\n",
                     name, ms * 1e6 / iters, phase_clk, (double)h[0] / 32.0, (double)h[1] / 32.0, ghz);
     else
@@ -394,13 +404,13 @@ inline int phase_probe() {
     std::printf("phase-probe: two groups of four waves per compute unit alternate between the matrix and the vector work of one\n"
                 "32-key x 64-query sub-tile at head_dim 64 (N(0,1) operands, no memory traffic), %d compute units\n", blocks);
     for (int rep = 0; rep < 2; rep++) {
-        if (run_phase<0, 0>("matrix phases only", blocks, out, clk, data)) return 2;
-        if (run_phase<1, 0>("matrix and vector phases", blocks, out, clk, data)) return 2;
+        if (run_phase<0, 2>("matrix phases only", blocks, out, clk, data)) return 2;
+        if (run_phase<1, 2>("matrix and vector phases", blocks, out, clk, data)) return 2;
         if (run_phase<0, 1>("matrix phases only", blocks, out, clk, data)) return 2;
         if (run_phase<1, 1>("matrix and vector phases", blocks, out, clk, data)) return 2;
-        if (run_phase<2, 0>("reference as a fifth k-step, no fma", blocks, out, clk, data)) return 2;
-        if (run_phase<3, 0>("row sums by v_add_f32", blocks, out, clk, data)) return 2;
-        if (run_phase<4, 0>("half the row-sum mfma, pk_add_f16", blocks, out, clk, data)) return 2;
+        if (run_phase<2, 2>("reference as a fifth k-step, no fma", blocks, out, clk, data)) return 2;
+        if (run_phase<3, 2>("row sums by v_add_f32", blocks, out, clk, data)) return 2;
+        if (run_phase<4, 2>("half the row-sum mfma, pk_add_f16", blocks, out, clk, data)) return 2;
     }
     (void)hipFree(out);
     (void)hipFree(clk);
