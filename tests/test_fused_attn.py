@@ -467,6 +467,35 @@ def test_very_long_ragged_sequence(gpu, R, H, causal):
         assert (zero - mean).abs().max().item() <= 1e-3
 
 
+@pytest.mark.parametrize("B,R,L,H", [(1, 3, 300, 64), (4, 16, 2048, 64), (2, 64, 1024, 128)])
+def test_non_finite_inputs_stay_where_the_oracle_puts_them(gpu, B, R, L, H):
+    """A NaN in one query row and an inf in one key row: the call returns, the rows the oracle
+    leaves finite match it, the rows it makes NaN are NaN, and the other heads do not change a bit."""
+    q, k, v = (_rand((B, L, R * H), 8800 + L + i) for i in range(3))
+    clean = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H).cpu()
+    q2, k2 = q.clone(), k.clone()
+    q2[0, 5, 3] = float("nan")                       # head 0, query 5
+    k2[B - 1, L - 2, H + 1] = float("inf")           # head 1 of the last batch, key L - 2
+    got = capi.forward(q2.to(gpu), k2.to(gpu), v.to(gpu), H).cpu()
+    # heads and batches that hold no non-finite input: bitwise unchanged
+    touched = torch.zeros(B, R, dtype=torch.bool)
+    touched[0, 0] = True
+    touched[B - 1, 1] = True
+    for b in range(B):
+        for h in range(R):
+            if not touched[b, h]:
+                assert torch.equal(got[b, :, h * H:(h + 1) * H], clean[b, :, h * H:(h + 1) * H]), (b, h)
+    for b, h in ((0, 0), (B - 1, 1)):
+        sl = slice(h * H, (h + 1) * H)
+        want = attention(q2[b:b + 1, :, sl], k2[b:b + 1, :, sl], v[b:b + 1, :, sl], H)[0]
+        mine = got[b, :, sl].float()
+        bad = ~torch.isfinite(want).all(dim=-1)
+        assert bad.any()
+        assert (~torch.isfinite(mine[bad])).any(dim=-1).all()
+        assert torch.isfinite(mine[~bad]).all()
+        assert (mine[~bad] - want[~bad]).abs().max().item() <= TOL
+
+
 # ---- every launch shape, plain and masked -------------------------------------------------------------
 
 def _check_pairs_tol(got, q, k, v, H, pairs, mask, tol):
