@@ -172,6 +172,9 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     if (q == nullptr || k == nullptr || v == nullptr || out == nullptr) return FA_ERR_NULL_POINTER;
     if (!fa_fwd_query(H)) return FA_ERR_BAD_HEAD_DIM;
     if (B < 1 || R < 1 || L < 1) return FA_ERR_BAD_SHAPE;
+    // the kernels track the row maximum of the raw scores, which is the maximum of the scaled ones
+    // only for a positive scale, and they divide the additive mask by the scale
+    if (!(scale > 0.f) || scale > 3.0e38f) return FA_ERR_BAD_SCALE;
     if (!strides_ok(in, H) || !strides_ok(os, H)) return FA_ERR_BAD_STRIDE;
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return FA_ERR_MISALIGNED;
     if (mask != nullptr && (reinterpret_cast<uintptr_t>(mask) & 1u) != 0) return FA_ERR_MISALIGNED;
@@ -227,6 +230,7 @@ const char* fa_strerror(int status) {
         case FA_ERR_MISALIGNED: return "fa_fwd: q, k, v and out must be 16-byte aligned";
         case FA_ERR_TOO_LARGE: return "fa_fwd: problem size exceeds the supported index range";
         case FA_ERR_BAD_FLAGS: return "fa_fwd_ex: unknown flag, or FA_FLAG_CAUSAL together with a mask";
+        case FA_ERR_BAD_SCALE: return "fa_fwd: scale must be finite and positive";
         default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));

@@ -33,6 +33,7 @@ extern "C" {
 #define FA_ERR_MISALIGNED (-5)
 #define FA_ERR_TOO_LARGE (-6)
 #define FA_ERR_BAD_FLAGS (-7)
+#define FA_ERR_BAD_SCALE (-8)
 
 #define FA_FLAG_CAUSAL 1
 #define FA_FLAG_BF16 2
@@ -51,6 +52,8 @@ extern "C" {
  *   - `mask` (nullable) is an additive fp16 [B, L, L] tensor shared by all heads and is
  *     applied to every key, not only to the first chunk.  Rows whose keys are all -inf
  *     produce zeros.
+ * `scale` is finite and > 0 (FA_ERR_BAD_SCALE otherwise); the reference fixes it at
+ * 1/sqrt(head_dim) (reference include/fused_attn.cuh:727).
  * B, R, L >= 1.  L*stride_l, R*stride_h and B*stride_b must stay below 2^62 elements and
  * stride_l must not exceed 2^24 elements (FA_ERR_TOO_LARGE otherwise).
  */

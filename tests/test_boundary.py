@@ -66,7 +66,8 @@ def test_status_codes_for_rejected_arguments():
     assert strided((L * R * H, H, R * H + 2), dense) == -4
     assert strided(packed, (2 ** 62 + 8, H, R * H)) == -6         # output extent beyond the index range
     assert strided(packed, dense, flags=8) == -7
-    for code in (-1, -2, -3, -4, -5, -6, -7):
+    assert status(scale=0.0) == -8 and status(scale=-0.125) == -8 and status(scale=float("nan")) == -8 and status(scale=float("inf")) == -8
+    for code in (-1, -2, -3, -4, -5, -6, -7, -8):
         assert "fa_fwd" in capi.strerror(code)
     assert capi.strerror(0) == "success"
 

@@ -496,6 +496,30 @@ def test_non_finite_inputs_stay_where_the_oracle_puts_them(gpu, B, R, L, H):
         assert (mine[~bad] - want[~bad]).abs().max().item() <= TOL
 
 
+@pytest.mark.parametrize("B,R,L,H", [(2, 3, 300, 64), (4, 16, 2048, 64), (2, 64, 1024, 128)])
+def test_scale_argument(gpu, B, R, L, H):
+    """The C ABI takes the softmax scale as an argument (the reference fixes it at 1/sqrt(head_dim)):
+    a tiny one gives the mean of the value rows, any other value equals the default scale on
+    queries multiplied by scale * sqrt(head_dim) (done in fp32 on the oracle's side)."""
+    q, k, v = (_rand((B, L, R * H), 9100 + L + i) for i in range(3))
+    dq, dk, dv = q.to(gpu), k.to(gpu), v.to(gpu)
+    flat = capi.forward(dq, dk, dv, H, scale=1e-9)
+    assert _max_err(flat, v.float().mean(dim=1, keepdim=True).expand(B, L, R * H)) <= 1e-3
+    for scale in (1.0 / H, 0.3, 1.0):
+        got, lse = capi.forward(dq, dk, dv, H, scale=scale, return_lse=True)
+        qs = q.float() * (scale * math.sqrt(H))
+        pairs = [(0, 0), (B - 1, R - 1)]
+        for b, h in pairs:
+            sl = slice(h * H, (h + 1) * H)
+            want = attention(qs[b:b + 1, :, sl], k[b:b + 1, :, sl], v[b:b + 1, :, sl], H)
+            assert _max_err(got[b:b + 1, :, sl], want) <= TOL, (scale, b, h)
+            want_lse = attention_lse(qs[b:b + 1, :, sl], k[b:b + 1, :, sl], H)[0, 0]
+            assert (lse[b, h].cpu() - want_lse).abs().max().item() <= 2e-3, (scale, b, h)
+    for bad in (0.0, -1.0, float("nan"), float("inf")):
+        with pytest.raises(capi.FusedAttnError):
+            capi.forward(dq, dk, dv, H, scale=bad)
+
+
 # ---- every launch shape, plain and masked -------------------------------------------------------------
 
 def _check_pairs_tol(got, q, k, v, H, pairs, mask, tol):
