@@ -386,6 +386,42 @@ def test_additive_mask_on_every_key_tile(gpu, L, H, offset):
     assert _max_err(got, want) <= TOL
 
 
+@pytest.mark.parametrize("B,R,L,H", [(2, 2, 200, 64), (4, 16, 2048, 64), (2, 40, 1024, 128)])
+def test_mask_of_finite_minimum_values(gpu, B, R, L, H):
+    """Masks as libraries commonly build them: the most negative fp16 number (-65504) instead of
+    -inf, here above the diagonal and on the padded keys at the end of the last batch entry."""
+    q, k, v = (_rand((B, L, R * H), 3650 + L + i) for i in range(3))
+    lowest = torch.finfo(torch.float16).min
+    mask = torch.full((L, L), lowest).triu(1).expand(B, L, L).clone()
+    mask[B - 1, :, L - 37:] = lowest
+    mask = mask.to(torch.float16)
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, mask=mask.to(gpu))
+    assert torch.isfinite(got.float()).all()
+    # the oracle with -inf in the same places: every row keeps at least key 0
+    hard = torch.where(mask == lowest, float("-inf"), 0.0)
+    _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R - 1)], mask=hard)
+
+
+@pytest.mark.parametrize("B,R,L,H", [(2, 2, 200, 64), (4, 16, 2048, 64), (2, 40, 1024, 128)])
+def test_subnormal_inputs(gpu, B, R, L, H):
+    """fp16 subnormals (below 6.1e-5) are operands like any other: values of that size come out
+    as their weighted mean, not as zero, and subnormal queries and keys give uniform weights."""
+    q, k, v = (_rand((B, L, R * H), 3680 + L + i) for i in range(3))
+    tiny_v = (v.float() * 2e-5).to(torch.float16)
+    assert (tiny_v.float().abs() < 6.1e-5).float().mean() > 0.9
+    got = capi.forward(q.to(gpu), k.to(gpu), tiny_v.to(gpu), H).float().cpu()
+    for b, h in [(0, 0), (B - 1, R - 1)]:
+        sl = slice(h * H, (h + 1) * H)
+        want = attention(q[b:b + 1, :, sl], k[b:b + 1, :, sl], tiny_v[b:b + 1, :, sl], H)
+        # compared in units of the values' own size; the output has fp16 subnormal spacing 6e-8
+        assert ((got[b:b + 1, :, sl] - want).abs().max().item()) / 2e-5 <= TOL + 6e-8 / 2e-5
+        assert got[b, :, sl].abs().max().item() > 0
+    tiny_q = (q.float() * 1e-5).to(torch.float16)
+    tiny_k = (k.float() * 1e-5).to(torch.float16)
+    flat = capi.forward(tiny_q.to(gpu), tiny_k.to(gpu), v.to(gpu), H)
+    assert _max_err(flat, v.float().mean(dim=1, keepdim=True).expand(B, L, R * H)) <= 1e-3
+
+
 def test_fully_masked_rows_give_zeros_not_nan(gpu):
     B, R, L, H = 1, 2, 100, 64
     q, k, v = (_rand((B, L, R * H), 3600 + i) for i in range(3))
