@@ -201,6 +201,32 @@ def test_views_in_the_bhld_layout_and_mismatched_strides(gpu):
         capi.forward(q.transpose(2, 3).contiguous().transpose(2, 3), k, v, H, layout="bhld")
 
 
+@pytest.mark.parametrize("R,L,H", [(2, 70, 64), (160, 600, 64), (80, 600, 128)])
+def test_row_pitch_at_the_limit(gpu, R, L, H):
+    """stride_l = 2^24 elements, the largest the library accepts (32 MiB between sequence
+    positions): q, k, v are column ranges of one [L, 2^24] buffer.  Bitwise the result of the
+    same call on contiguous copies, through the four-wave and the eight-wave kernel."""
+    F = R * H
+    pitch = 1 << 24
+    buf = torch.empty((L, pitch), dtype=torch.float16, device=gpu)      # 2.3 GB / 20 GB, mostly untouched
+    buf[:, :3 * F] = _rand((L, 3 * F), 4100 + L).to(gpu)
+    q, k, v = (buf[:, i * F:(i + 1) * F].unsqueeze(0) for i in range(3))
+    assert q.stride()[1:] == (pitch, 1)
+    want, want_lse = capi.forward(q.contiguous(), k.contiguous(), v.contiguous(), H, return_lse=True)
+    got, got_lse = capi.forward(q, k, v, H, return_lse=True)
+    assert torch.equal(got, want) and torch.equal(got_lse, want_lse)
+    assert torch.equal(capi.forward(q, k, v, H, causal=True),
+                       capi.forward(q.contiguous(), k.contiguous(), v.contiguous(), H, causal=True))
+    _check_pairs(got.cpu(), q.contiguous().cpu(), k.contiguous().cpu(), v.contiguous().cpu(), H, [(0, 0), (0, R - 1)])
+    # one element more is rejected
+    with pytest.raises(capi.FusedAttnError, match="index range"):
+        status = capi.load_library().fa_fwd_strided(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), None, got.data_ptr(), None, 1, R, L, H,
+            L * pitch, H, pitch + 8, L * F, H, F, 0.125, 0, None)
+        capi._check(status)
+    del buf
+
+
 def test_runs_on_the_current_stream_and_is_deterministic(gpu):
     import fused_attn
 
