@@ -241,6 +241,30 @@ def test_runs_on_the_current_stream_and_is_deterministic(gpu):
     assert torch.equal(first, second)
 
 
+def test_concurrent_calls_from_host_threads(gpu):
+    """The library keeps no state between calls except a mutex-guarded list of kernels whose LDS
+    limit it has raised: four host threads launching different shapes on streams of their own
+    get the results of the same calls made one after the other."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    shapes = [(2, 3, 300, 64, False), (4, 16, 2048, 64, False), (2, 40, 1024, 128, True), (1, 24, 777, 32, False)]
+    inputs = [tuple(_rand((B, L, R * H), 4300 + L + i).to(gpu) for i in range(3)) for B, R, L, H, _ in shapes]
+    serial = [capi.forward(*inputs[i], shapes[i][3], causal=shapes[i][4]) for i in range(len(shapes))]
+    torch.cuda.synchronize()
+
+    def work(i):
+        stream = torch.cuda.Stream(device=gpu)
+        outs = []
+        with torch.cuda.stream(stream):
+            for _ in range(20):
+                outs.append(capi.forward(*inputs[i], shapes[i][3], causal=shapes[i][4]))
+        stream.synchronize()
+        return all(torch.equal(o, serial[i]) for o in outs)
+
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        assert all(pool.map(work, range(len(shapes))))
+
+
 # ---- closed forms (no oracle involved) ---------------------------------------------------------------
 
 @pytest.mark.parametrize("L", [1000, 3073])
