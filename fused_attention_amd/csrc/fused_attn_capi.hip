@@ -27,9 +27,9 @@ struct Shape {
 //           workgroup, one resident per compute unit (head_dim <= 64 only: with head_dim 128 a
 //           64-row wave would need the whole register file of a SIMD);
 //   {8, 1}  the same kernel with 32-row waves, 256 queries per workgroup: the only ping-pong
-//           shape of head_dim 128 (one resident per compute unit); with head_dim <= 64 two are
-//           resident per compute unit and it serves the grids that {8, 2} fills badly (without
-//           mask only: the causal and the additive-mask variants do not fit 128 registers);
+//           shape of head_dim 128 (one resident per compute unit); with head_dim <= 64 it serves
+//           the grids that {8, 2} fills badly (without mask two are resident per compute unit;
+//           the causal and the additive-mask variants do not fit 128 registers and run one);
 //   {4, 1}  four 32-row waves, 128 queries per workgroup, three (head_dim <= 64) or two
 //           (head_dim 128) resident per compute unit: more, smaller workgroups for small problems.
 int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -64,11 +64,21 @@ Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask, bool
     const bool pingpong = wgs8 >= 2 * kNumCu ? usage8 >= 614 : usage8 >= (wgs8 <= kNumCu ? 614 : 717);
     if (H > 64) return pingpong ? Shape{8, 1} : Shape{4, 1};
     if (pingpong) return {8, 2};
-    // 256-query ping-pong workgroups, two per compute unit: per compute unit they run at 0.93 of
-    // the 512-query ones and 1.1 to 1.25 times as fast as the four-wave kernel, but they need 160
-    // or more workgroups to beat the latter's finer grain (sweep of 22 mid-size shapes on MI355X).
-    if (has_mask || causal) return {4, 1};
-    return heads * ceil_div(L, 256) >= 160 ? Shape{8, 1} : Shape{4, 1};
+    // 256-query ping-pong workgroups.  Thresholds from sweeps of mid-size shapes on MI355X.
+    // Causal (a workgroup takes a pair of 256-query tiles, one resident per compute unit): 4 to
+    // 21 % faster than the four-wave kernel when the pairs fill 60 % or more of a single round,
+    // slower on emptier or on several rounds.
+    if (causal)
+        return heads * ceil_div(L, 512) <= kNumCu && usage(heads, L, 512, kNumCu) >= 614 ? Shape{8, 1} : Shape{4, 1};
+    // Additive mask (one resident per compute unit): up to 18 % faster than the four-wave kernel,
+    // whose masked loop is not pipelined, from 160 workgroups on, unless a quarter or more of the
+    // query rows of a head's workgroups do not exist.
+    const int64_t per_head = ceil_div(L, 256);
+    if (has_mask) return heads * per_head >= 160 && 4 * L >= 3 * per_head * 256 ? Shape{8, 1} : Shape{4, 1};
+    // Plain, two per compute unit: per compute unit they run at 0.93 of the 512-query ones and
+    // 1.1 to 1.25 times as fast as the four-wave kernel, but they need 160 or more workgroups to
+    // beat the latter's finer grain.
+    return heads * per_head >= 160 ? Shape{8, 1} : Shape{4, 1};
 }
 
 // Dynamic LDS above 64 KiB has to be opted into per kernel function and per device: done on the
@@ -125,7 +135,7 @@ hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) 
         else if constexpr (MODE == fa::kPlain)
             return launch_pingpong<H, 8, 1, 4, MODE, BF>(p, stream);
         else
-            return hipErrorInvalidValue;     // pick_shape never asks for this
+            return launch_pingpong<H, 8, 1, 2, MODE, BF>(p, stream);
     }
     // four 32-row waves; three per SIMD where the registers allow it
     if constexpr (H > 64 || MODE == fa::kAdditive)

@@ -697,6 +697,8 @@ def test_eight_wave_kernel_reference_lag(gpu, B, R, L, H, step_log2):
     (2, 64, 1024, 128),     # head_dim 128, four tiles of 256 queries
     (4, 64, 1250, 128),     # head_dim 128, five tiles, ragged end
     (8, 64, 512, 64), (3, 100, 300, 32),     # four-wave workgroups
+    (8, 12, 1024, 64), (1, 20, 4096, 64),    # eight 32-row waves: pairs of 256-query tiles filling most of one round
+    (3, 16, 2000, 32), (16, 16, 500, 16),    # ... at the smaller head dims, with ragged ends
 ])
 def test_causal_on_large_grids(gpu, B, R, L, H):
     q, k, v = (_rand((B, L, R * H), 3950 + L + i) for i in range(3))
@@ -717,6 +719,7 @@ def test_causal_on_large_grids(gpu, B, R, L, H):
     (4, 40, 704, 128),                                           # ... head_dim 128, ragged end
     (2, 64, 1023, 64),                                           # element-wise mask loads (L % 4 != 0)
     (4, 40, 700, 128),                                           # 8-byte mask loads (L % 8 != 0)
+    (2, 12, 2048, 64), (1, 500, 256, 64), (2, 12, 2040, 16), (1, 40, 2104, 32),   # eight 32-row waves, 256-query workgroups
 ])
 def test_additive_mask_on_large_grids(gpu, B, R, L, H):
     q, k, v = (_rand((B, L, R * H), 3970 + L + i) for i in range(3))
