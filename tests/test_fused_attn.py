@@ -754,6 +754,7 @@ BF16_TOL = 2e-2   # bf16 keeps 8 significant bits: the output rounding alone is 
     (2, 64, 1024, 128, False), (2, 64, 1024, 128, True),
     (2, 8, 1000, 64, False),
     (2, 8, 3073, 64, False),                                  # eight 32-row waves, two workgroups per CU
+    (8, 12, 1024, 64, True), (3, 16, 2000, 32, True),         # ... causal, one workgroup per CU
 ])
 def test_bf16_inputs(gpu, B, R, L, H, causal):
     q, k, v = (_rand((B, L, R * H), 4200 + L + i).to(torch.bfloat16) for i in range(3))
@@ -770,7 +771,7 @@ def test_bf16_inputs(gpu, B, R, L, H, causal):
         assert ((lse[b, h].cpu() - want_lse).abs() / (1 + want_lse.abs())).max().item() <= 2e-3
 
 
-@pytest.mark.parametrize("B,R,L,H", [(2, 2, 200, 64), (8, 64, 512, 64)])
+@pytest.mark.parametrize("B,R,L,H", [(2, 2, 200, 64), (8, 64, 512, 64), (2, 12, 2048, 64), (2, 12, 2040, 16)])
 def test_bf16_additive_mask_and_closed_forms(gpu, B, R, L, H):
     q, k, v = (_rand((B, L, R * H), 4300 + i).to(torch.bfloat16) for i in range(3))
     g = torch.Generator().manual_seed(4310)
