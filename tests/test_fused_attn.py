@@ -720,6 +720,8 @@ def test_causal_on_large_grids(gpu, B, R, L, H):
     (2, 64, 1023, 64),                                           # element-wise mask loads (L % 4 != 0)
     (4, 40, 700, 128),                                           # 8-byte mask loads (L % 8 != 0)
     (2, 12, 2048, 64), (1, 500, 256, 64), (2, 12, 2040, 16), (1, 40, 2104, 32),   # eight 32-row waves, 256-query workgroups
+    (1, 40, 2048, 128), (4, 40, 512, 128),   # head_dim 128: 256-query workgroups on a part-filled second round
+    (4, 12, 1536, 64),                       # 64-row waves on a lone round filled to 56 %
 ])
 def test_additive_mask_on_large_grids(gpu, B, R, L, H):
     q, k, v = (_rand((B, L, R * H), 3970 + L + i) for i in range(3))
