@@ -65,6 +65,9 @@ struct FwdParams {
                            // that (rounded up) when a causal workgroup takes a pair of query tiles
     int total_wgs;         // B * R * n_qtiles
     int wgs_per_xcd;       // ceil(total_wgs / 8)
+    int heads_per_xcd;     // causal eight-wave launches: 0 = every workgroup takes the pair of query tiles
+                           // (t, n - 1 - t) of one head; > 0 = resident grid, the heads of an XCD's
+                           // workgroups (B * R / 8 of them) dealt out tile by tile, see the kernel
     float scale_log2e;     // scale * log2(e)
 };
 
@@ -74,6 +77,7 @@ constexpr int kNumXcd = 8;
 constexpr int kPlain = 0;    // no mask: software-pipelined loop
 constexpr int kAdditive = 1; // additive [B, L, L] mask
 constexpr int kCausal = 2;   // key index <= query index, key tiles above the diagonal skipped
+constexpr int kCausalDealt = 3;   // eight-wave kernel only: causal with the query tiles dealt out to a resident grid
 
 template <int H>
 struct Geometry {

@@ -699,6 +699,8 @@ def test_eight_wave_kernel_reference_lag(gpu, B, R, L, H, step_log2):
     (8, 64, 512, 64), (3, 100, 300, 32),     # four-wave workgroups
     (8, 12, 1024, 64), (1, 20, 4096, 64),    # eight 32-row waves: pairs of 256-query tiles filling most of one round
     (3, 16, 2000, 32), (16, 16, 500, 16),    # ... at the smaller head dims, with ragged ends
+    (2, 40, 2048, 128), (2, 40, 4096, 64),   # 320 pairs would leave a second round three quarters empty: tiles dealt out to a resident grid
+    (2, 40, 2300, 128), (2, 48, 5000, 32),   # ... with an odd number of tiles and ragged ends
 ])
 def test_causal_on_large_grids(gpu, B, R, L, H):
     q, k, v = (_rand((B, L, R * H), 3950 + L + i) for i in range(3))
