@@ -48,7 +48,8 @@ int64_t usage(int64_t heads, int64_t L, int64_t rows, int64_t slots) {
 
 // Causal launches of the eight-wave kernel.  Query tile t of a head costs t + 1 key blocks.  The
 // plain schedule gives every workgroup the pair (t, n - 1 - t), n + 1 blocks, and the grid runs
-// ceil(pairs / 256) rounds of them; a last round that is mostly empty costs as much as a full one.
+// ceil(pairs / 256) rounds of them; a last round that is mostly empty costs as much as a full one,
+// and in a lone part-filled round the idle compute units could have taken the small tiles.
 // The dealt schedule (kernel: p.heads_per_xcd > 0) keeps 32 workgroups resident per XCD and deals
 // the tiles of the XCD's heads out in descending cost, serpentine over the workgroups; it needs
 // B * R to be a multiple of 8 so that the XCDs carry equal loads.  Time in key blocks of the
@@ -65,7 +66,7 @@ CausalPlan plan_causal(int64_t heads, int64_t n, int64_t H) {
     constexpr int kPerXcd = kNumCu / fa::kNumXcd;
     // head_dim below 64: dealing the tiles out spreads an XCD's workgroups over more heads at a
     // time than its L2 holds K and V for, and measures slower than the part-filled round
-    if (H < 64 || heads % fa::kNumXcd != 0 || pairs <= kNumCu) return paired;
+    if (H < 64 || heads % fa::kNumXcd != 0) return paired;
     const int64_t hx = heads / fa::kNumXcd;
     const int64_t items = hx * n;
     if (items > (int64_t)1 << 22) return paired;     // the walk below is linear in the items
@@ -175,18 +176,20 @@ hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
 
 template <int H, int MODE, bool BF>
 hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) {
-    // the dealt causal schedule exists for the 512-query (256 at head_dim 128) workgroups only
+    // the dealt causal schedule exists for the eight-wave kernel at head_dim 64 and 128 only
+    // (plan_causal never asks for it elsewhere)
     constexpr int BASE = MODE == fa::kCausalDealt ? fa::kCausal : MODE;
+    if (MODE == fa::kCausalDealt && (sh.waves != 8 || H < 64)) return hipErrorInvalidValue;
     // the ping-pong kernel for the eight-wave shapes
     if (sh.waves == 8) {
         if constexpr (H > 64)
             return launch_pingpong<H, 8, 1, 2, MODE, BF>(p, stream);
         else if (sh.nqb == 2)
-            return launch_pingpong<H, 8, 2, 2, H < 64 ? BASE : MODE, BF>(p, stream);   // never dealt below head_dim 64
+            return launch_pingpong<H, 8, 2, 2, H < 64 ? BASE : MODE, BF>(p, stream);
         else if constexpr (MODE == fa::kPlain)
             return launch_pingpong<H, 8, 1, 4, MODE, BF>(p, stream);
         else
-            return launch_pingpong<H, 8, 1, 2, BASE, BF>(p, stream);
+            return launch_pingpong<H, 8, 1, 2, H < 64 ? BASE : MODE, BF>(p, stream);
     }
     // four 32-row waves; three per SIMD where the registers allow it
     if constexpr (H > 64 || MODE == fa::kAdditive)

@@ -701,6 +701,7 @@ def test_eight_wave_kernel_reference_lag(gpu, B, R, L, H, step_log2):
     (3, 16, 2000, 32), (16, 16, 500, 16),    # ... at the smaller head dims, with ragged ends
     (2, 40, 2048, 128), (2, 40, 4096, 64),   # 320 pairs would leave a second round three quarters empty: tiles dealt out to a resident grid
     (2, 40, 2300, 128), (2, 48, 5000, 32),   # ... with an odd number of tiles and ragged ends
+    (1, 40, 2048, 128), (1, 40, 4000, 64),   # ... fewer pairs than compute units: single tiles spread over all of them
 ])
 def test_causal_on_large_grids(gpu, B, R, L, H):
     q, k, v = (_rand((B, L, R * H), 3950 + L + i) for i in range(3))
