@@ -11,7 +11,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libfused_attn_gfx950.so")
 
 # every symbol include/fused_attn.h declares
-EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_strided", "fa_fwd_query", "fa_strerror", "fa_fwd_timed")
+EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_strided", "fa_fwd_plan", "fa_fwd_query", "fa_strerror", "fa_fwd_timed")
 FLAG_CAUSAL = 1
 FLAG_BF16 = 2
 
@@ -48,6 +48,8 @@ def load_library():
     lib.fa_fwd_strided.restype = ctypes.c_int
     lib.fa_fwd_timed.argtypes = fwd_args + [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
     lib.fa_fwd_timed.restype = ctypes.c_int
+    lib.fa_fwd_plan.argtypes = [i64, i64, i64, i64, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int)]
+    lib.fa_fwd_plan.restype = ctypes.c_int
     lib.fa_fwd_query.argtypes = [i64]
     lib.fa_fwd_query.restype = ctypes.c_int
     lib.fa_strerror.argtypes = [ctypes.c_int]
@@ -63,6 +65,14 @@ def strerror(status):
 def _check(status):
     if status != 0:
         raise FusedAttnError(status, strerror(status))
+
+
+def launch_plan(B, R, L, H, causal=False, has_mask=False):
+    """What fa_fwd_plan reports for a problem, as a dict.  Needs no GPU."""
+    out = (ctypes.c_int * 6)()
+    _check(load_library().fa_fwd_plan(B, R, L, H, FLAG_CAUSAL if causal else 0, 1 if has_mask else 0, out))
+    keys = ("waves", "rows_per_wave", "workgroups", "working", "per_head", "heads_per_xcd")
+    return dict(zip(keys, out))
 
 
 def fwd_raw(q_ptr, k_ptr, v_ptr, mask_ptr, out_ptr, B, R, L, H, stride_b, stride_h, stride_l,

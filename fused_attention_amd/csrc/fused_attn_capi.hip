@@ -335,6 +335,28 @@ int fa_fwd_strided(const void* q, const void* k, const void* v, const void* mask
     return static_cast<int>(e);
 }
 
+int fa_fwd_plan(int64_t B, int64_t R, int64_t L, int64_t H, int flags, int has_mask, int* plan) {
+    if (plan == nullptr) return FA_ERR_NULL_POINTER;
+    if ((flags & ~(FA_FLAG_CAUSAL | FA_FLAG_BF16)) != 0) return FA_ERR_BAD_FLAGS;
+    const bool causal = (flags & FA_FLAG_CAUSAL) != 0;
+    if (causal && has_mask) return FA_ERR_BAD_FLAGS;
+    // validate() only looks at the pointers' alignment
+    void* const fake = reinterpret_cast<void*>(static_cast<uintptr_t>(4096));
+    fa::FwdParams p;
+    Shape shape{4, 1};
+    const Strides dense{L * R * H, H, R * H};
+    const int rc = validate(fake, fake, fake, has_mask ? fake : nullptr, fake, B, R, L, H, dense, dense, &p, 1.0f,
+                            &shape, causal, nullptr);
+    if (rc != FA_OK) return rc;
+    plan[0] = shape.waves;
+    plan[1] = 32 * shape.nqb;
+    plan[2] = p.wgs_per_xcd * fa::kNumXcd;
+    plan[3] = p.total_wgs;
+    plan[4] = p.n_qtiles;
+    plan[5] = p.heads_per_xcd;
+    return FA_OK;
+}
+
 int fa_fwd_ex(const void* q, const void* k, const void* v, const void* mask, void* out, void* lse,
               int64_t B, int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h,
               int64_t stride_l, float scale, int flags, void* stream) {

@@ -99,6 +99,18 @@ int fa_fwd_strided(const void* q, const void* k, const void* v, const void* mask
                    float scale, int flags, void* stream);
 
 /*
+ * The launch the library would make for a problem, without making it (no GPU is touched): for
+ * tests of the launcher and for tuning.  has_mask != 0 stands for an additive mask with 16-byte
+ * aligned rows.  Fills plan[0..5] with: wave64s per workgroup; query rows per wave; workgroups
+ * launched; workgroups that do work (the rest exit at once); workgroups per (batch, head), or
+ * pairs of query tiles per head for a causal launch of the eight-wave kernel; 0, or, when the
+ * query tiles of a causal launch are dealt out to a resident grid, the heads per XCD.
+ * The reference has no counterpart (its grid is fixed at (B, L / chunk_size, R),
+ * reference include/fused_attn.cuh:872-883).
+ */
+int fa_fwd_plan(int64_t B, int64_t R, int64_t L, int64_t H, int flags, int has_mask, int* plan);
+
+/*
  * 1 if fa_fwd accepts this head_dim, else 0.  Counterpart of the compile-time
  * (head_dim, chunk_size) dispatch table (reference src/fused_attn_extention.cu:72-111).
  */

@@ -72,6 +72,68 @@ def test_status_codes_for_rejected_arguments():
     assert capi.strerror(0) == "success"
 
 
+def _items_of_plan(plan, heads, L, causal):
+    """Replays how the kernels turn a workgroup index into (head, query tile) items
+    (fwd_kernel and fwd_kernel_pingpong in fused_attn_kernel_impl.inc) for a launch plan."""
+    rows = plan["waves"] * plan["rows_per_wave"]
+    tiles = -(-L // rows)
+    per_xcd = plan["workgroups"] // 8
+    items = []
+    for wg in range(plan["workgroups"]):
+        logical = (wg % 8) * per_xcd + wg // 8
+        if logical >= plan["working"]:
+            continue
+        if plan["heads_per_xcd"] > 0:                      # causal, tiles dealt out to a resident grid
+            w, rnd = wg // 8, 0
+            while True:
+                j = rnd * per_xcd + (per_xcd - 1 - w if rnd & 1 else w)
+                if j >= plan["heads_per_xcd"] * tiles:
+                    break
+                items.append((wg % 8 + 8 * (j % plan["heads_per_xcd"]), tiles - 1 - j // plan["heads_per_xcd"]))
+                rnd += 1
+        elif causal and plan["waves"] == 8:                # causal, a pair of tiles per workgroup
+            head, slot = divmod(logical, plan["per_head"])
+            items.append((head, tiles - 1 - slot))
+            if 2 * slot != tiles - 1:
+                items.append((head, slot))
+        else:
+            head, slot = divmod(logical, plan["per_head"])
+            items.append((head, tiles - 1 - slot if causal else slot))
+    return items, tiles
+
+
+def test_every_launch_plan_covers_every_query_tile_once():
+    """The launcher's grid and schedule parameters against the kernels' decoding of them, on the
+    CPU: every (head, query tile) exactly once, no index out of range, for plain, masked and
+    causal launches over shapes that reach every branch of the shape and schedule choice."""
+    import random
+
+    rng = random.Random(20261127)
+    shapes = [(4, 16, 4096, 64), (1, 32, 16384, 128), (4, 40, 2048, 128), (8, 12, 1024, 64), (2, 8, 3073, 64),
+              (2, 40, 2048, 128), (2, 40, 4096, 64), (2, 40, 2300, 128), (1, 40, 2048, 128), (1, 40, 4000, 64),
+              (2, 48, 5000, 32), (1, 20, 4096, 64), (16, 16, 500, 16), (1, 1, 1, 16), (3, 5, 7, 32), (1, 500, 256, 64),
+              (1, 8, 65537, 64), (64, 12, 128, 64), (1, 96, 100000, 128)]
+    for _ in range(400):
+        H = rng.choice([16, 32, 64, 128])
+        L = rng.choice([rng.randint(1, 300), rng.randint(301, 3000), rng.randint(3001, 20000)])
+        heads = rng.choice([1, 3, 8, 12, 16, 20, 24, 40, 48, 64, 80, 96, 120, 160, 256, 320, 640])
+        B = rng.choice([b for b in (1, 2, 4, 8) if heads % b == 0])
+        shapes.append((B, heads // B, L, H))
+    dealt = 0
+    for B, R, L, H in shapes:
+        for causal, has_mask in ((False, False), (True, False), (False, True)):
+            if has_mask and L % 8:
+                continue
+            plan = capi.launch_plan(B, R, L, H, causal=causal, has_mask=has_mask)
+            assert plan["waves"] in (4, 8) and plan["rows_per_wave"] in (32, 64) and plan["workgroups"] % 8 == 0
+            assert plan["heads_per_xcd"] == 0 or (causal and plan["waves"] == 8 and H >= 64 and (B * R) % 8 == 0)
+            items, tiles = _items_of_plan(plan, B * R, L, causal)
+            assert len(items) == B * R * tiles, (B, R, L, H, causal, has_mask, plan)
+            assert set(items) == {(h, t) for h in range(B * R) for t in range(tiles)}, (B, R, L, H, causal, has_mask, plan)
+            dealt += plan["heads_per_xcd"] > 0
+    assert dealt > 10          # the dealt schedule was among the plans
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(capi, "_lib", None)
     monkeypatch.setattr(capi, "LIB_PATH", os.path.join(REPO, "does_not_exist.so"))
