@@ -134,6 +134,31 @@ def test_every_launch_plan_covers_every_query_tile_once():
     assert dealt > 10          # the dealt schedule was among the plans
 
 
+def test_benchmark_workloads_take_the_kernels_the_documentation_names():
+    def plan(B, R, L, H, **kw):
+        p = capi.launch_plan(B, R, L, H, **kw)
+        return p["waves"], p["rows_per_wave"], p["heads_per_xcd"] > 0
+
+    assert plan(4, 16, 4096, 64) == (8, 64, False)                       # c3: 512 workgroups of 512 queries
+    assert plan(1, 32, 16384, 128) == (8, 32, False)                     # c4
+    assert plan(4, 40, 2048, 128) == (8, 32, False)                      # README shape
+    assert plan(8, 12, 1024, 64) == (8, 64, False)                       # c2
+    assert plan(2, 8, 3073, 64) == (8, 32, False)                        # c5b: 256-query workgroups
+    assert plan(1, 4, 256, 64) == (4, 32, False)                         # c1
+    assert plan(2, 8, 1000, 64) == (4, 32, False)                        # c5a
+    assert plan(4, 16, 4096, 64, causal=True) == (8, 64, False)          # one whole round of pairs
+    assert plan(1, 32, 16384, 128, causal=True) == (8, 32, False)        # four whole rounds of pairs
+    assert plan(4, 40, 2048, 128, causal=True) == (8, 32, True)          # 2.5 rounds of pairs: dealt
+    assert plan(2, 40, 4096, 64, causal=True) == (8, 64, True)
+    assert plan(2, 48, 5000, 32, causal=True) == (8, 64, False)          # never dealt below head_dim 64
+    assert plan(8, 12, 1024, 64, causal=True)[:2] == (8, 32)             # pairs of 256-query tiles
+    assert plan(2, 12, 2048, 64, causal=True) == (4, 32, False)
+    assert plan(4, 16, 4096, 64, has_mask=True) == (8, 64, False)
+    assert plan(1, 40, 2048, 128, has_mask=True) == (8, 32, False)
+    assert plan(2, 12, 2048, 64, has_mask=True) == (8, 32, False)
+    assert plan(64, 12, 128, 64, has_mask=True) == (4, 32, False)
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(capi, "_lib", None)
     monkeypatch.setattr(capi, "LIB_PATH", os.path.join(REPO, "does_not_exist.so"))
