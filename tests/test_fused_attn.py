@@ -160,6 +160,7 @@ def test_native_bhld_layout_matches_packed_layout(gpu):
 @pytest.mark.parametrize("B,R,L,H,mode", [
     (2, 3, 200, 64, "plain"), (1, 2, 333, 128, "plain"), (2, 4, 130, 16, "plain"), (3, 2, 257, 32, "causal"),
     (1, 2, 200, 64, "mask"), (4, 16, 2048, 64, "plain"), (1, 32, 2048, 128, "causal"), (2, 80, 512, 64, "plain"),
+    (1, 40, 2048, 128, "causal"),
 ])
 def test_views_into_a_packed_qkv_tensor(gpu, B, R, L, H, mode):
     """q, k, v as slices of one [B, L, 3, R*H] projection output and a dense output of its own
@@ -760,6 +761,7 @@ BF16_TOL = 2e-2   # bf16 keeps 8 significant bits: the output rounding alone is 
     (2, 8, 1000, 64, False),
     (2, 8, 3073, 64, False),                                  # eight 32-row waves, two workgroups per CU
     (8, 12, 1024, 64, True), (3, 16, 2000, 32, True),         # ... causal, one workgroup per CU
+    (2, 40, 2048, 128, True), (1, 40, 4000, 64, True),        # causal, query tiles dealt out to a resident grid
 ])
 def test_bf16_inputs(gpu, B, R, L, H, causal):
     q, k, v = (_rand((B, L, R * H), 4200 + L + i).to(torch.bfloat16) for i in range(3))
