@@ -8,7 +8,7 @@ evaluation of the same workload timed on the host cores over a bounded sample of
 pairs.  Counterpart of the reference's benchmark (reference tests/benchmark_fused_attn.py:8-45),
 which prints wall-clock milliseconds of 128 naive and 128 fused launches.
 
-usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5a|c5b|readme]
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5a|c5b|readme] [--causal]
 """
 import argparse
 import json
@@ -71,6 +71,9 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="c3")
+    ap.add_argument("--causal", action="store_true",
+                    help="the causal extension of the C ABI instead of the reference's non-causal forward: "
+                         "counts the flops of the keys at or below the diagonal, no CPU baseline")
     ap.add_argument("--calibration-copy-mib", type=int, default=1024,
                     help="size of the plain copy run before the timed region (0 disables it)")
     ap.add_argument("--cpu-budget-s", type=float, default=15.0,
@@ -104,24 +107,43 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    if args.causal:
+        out = torch.empty_like(qd)
+
+        def step():
+            return capi.forward(qd, kd, vd, w.H, out=out, causal=True)
+    else:
+        def step():
+            return fused_attn.attention_forward(w.H, chunk, qd, kd, vd)
+
     for _ in range(args.warmup):
-        out = fused_attn.attention_forward(w.H, chunk, qd, kd, vd)
+        out = step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        out = fused_attn.attention_forward(w.H, chunk, qd, kd, vd)
+        out = step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
 
     # Kernel duration: HIP events on the launch stream around back-to-back launches.
-    kernel_ms = capi.forward_timed(qd, kd, vd, w.H, out, iters=args.steps)
+    if args.causal:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        kernel_ms = e0.elapsed_time(e1) / args.steps
+    else:
+        kernel_ms = capi.forward_timed(qd, kd, vd, w.H, out, iters=args.steps)
 
-    flop = workloads.flops(w)
+    # causal: query i attends to i + 1 keys
+    flop = 2.0 * w.B * w.R * w.L * (w.L + 1) * w.H if args.causal else workloads.flops(w)
     value = flop / (ms_per_step * 1e-3) / 1e12
     achieved = flop / (kernel_ms * 1e-3) / 1e12
     line = {
-        "metric": "fused attn fwd TFLOP/s (4*B*R*L^2*H)",
+        "metric": "fused attn fwd causal TFLOP/s (2*B*R*L*(L+1)*H)" if args.causal else "fused attn fwd TFLOP/s (4*B*R*L^2*H)",
         "value": value,
         "unit": "TFLOP/s",
         "pct_of_fp16_mfma_peak": 100.0 * value / PEAK_TFLOPS_FP16,
@@ -135,8 +157,9 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {
-            "workload": "%s: B=%d R=%d L=%d H=%d non-causal, fp16 N(0,%g) seeded on the host, "
-                        "fed as [B, L, R*H]" % (w.name, w.B, w.R, w.L, w.H, w.q_std),
+            "workload": "%s: B=%d R=%d L=%d H=%d %s, fp16 N(0,%g) seeded on the host, "
+                        "fed as [B, L, R*H]" % (w.name, w.B, w.R, w.L, w.H, "causal" if args.causal else "non-causal",
+                                                w.q_std),
             "flop_per_step": flop,
             "bytes_per_step": workloads.io_bytes(w),
         },
@@ -146,11 +169,11 @@ def main():
             "peak": PEAK_TFLOPS_FP16,
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_TFLOPS_FP16,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
+            "traffic": None if args.causal else MEASURED_TRAFFIC_BYTES.get(w.name),
             "kernel_ms": kernel_ms,
         },
     }
-    if args.cpu_budget_s > 0:
+    if args.cpu_budget_s > 0 and not args.causal:
         line["cpu_baseline"] = cpu_baseline(w, q, k, v, out, args.cpu_budget_s)
     print(json.dumps(line))
 
