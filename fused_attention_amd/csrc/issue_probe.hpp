@@ -228,7 +228,8 @@ inline int issue_probe() {
 // VWORK selects the work: 0 matrix phases only, 1 the kernel's split, and three splits the kernel
 // does not use, timed for comparison: 2 the reference folded into QK^T as a fifth k-step (no fma
 // in the vector phase), 3 row sums by v_add_f32 (no row-sum MFMAs), 4 pairs of packed
-// probabilities added in fp16 first (half the row-sum MFMAs).
+// probabilities added in fp16 first (half the row-sum MFMAs), 5 the kernel's split with the products
+// computed as 16x16 tiles (v_mfma_f32_16x16x32_f16, twice as many instructions of half the size).
 // STAMPS selects the clock readings: 0 none, 1 around every barrier (work per kind of phase; the
 // readings themselves add about 250 clocks to a phase), 2 two readings around the last 1024
 // phases (clocks per phase and shader clock of the undisturbed loop).
@@ -277,8 +278,35 @@ __global__ __launch_bounds__(512) void phase_kernel(float* out, long long* clk, 
                                              : u4v{pk[n][4 * t], pk[n][4 * t + 1], pk[n][4 * t + 2], pk[n][4 * t + 3]};
                     l[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[7], __builtin_bit_cast(h8, w), l[n], 0, 0, 0);
                 }
+            if (VWORK == 5) {
+                // the same products as 16x16 tiles: 16 instructions of 32 k for QK^T (8 tiles of S^T,
+                // two k-steps over head_dim 64), 16 for PV (16 tiles of O^T, one k-step over the 32 keys)
 #pragma unroll
-            for (int kk = 0; kk < (VWORK == 2 ? 5 : 4); kk++)
+                for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                    for (int n = 0; n < 2; n++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const f4v z = {0.f, 0.f, 0.f, 0.f};
+                            const f4v acc = {s[n][4 * i], s[n][4 * i + 1], s[n][4 * i + 2], s[n][4 * i + 3]};
+                            const f4v r = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[kk * 2 + (i & 1)], q[(kk * 2 + n) * 2 + (i >> 1)],
+                                                                                 kk == 0 ? z : acc, 0, 0, 0);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) s[n][4 * i + e] = r[e];
+                        }
+#pragma unroll
+                for (int t = 0; t < 16; t++) {
+                    const int n = t & 1, db = (t >> 1) & 1, i = t >> 2;
+                    const u4v w = {pk[n][4 * (i & 1)], pk[n][4 * (i & 1) + 1], pk[n][4 * (i & 1) + 2], pk[n][4 * (i & 1) + 3]};
+                    f16v& oo = o[db * 2 + n];
+                    const f4v acc = {oo[4 * i], oo[4 * i + 1], oo[4 * i + 2], oo[4 * i + 3]};
+                    const f4v r = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[4 + db * 2 + (i >> 1)], __builtin_bit_cast(h8, w), acc, 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) oo[4 * i + e] = r[e];
+                }
+            }
+#pragma unroll
+            for (int kk = 0; kk < (VWORK == 5 ? 0 : VWORK == 2 ? 5 : 4); kk++)
 #pragma unroll
                 for (int n = 0; n < 2; n++) {
                     f16v z;
@@ -287,7 +315,7 @@ __global__ __launch_bounds__(512) void phase_kernel(float* out, long long* clk, 
                                                                   kk == 0 ? z : s[n], 0, 0, 0);
                 }
 #pragma unroll
-            for (int t = 0; t < 2; t++)
+            for (int t = 0; t < (VWORK == 5 ? 0 : 2); t++)
 #pragma unroll
                 for (int db = 0; db < 2; db++)
 #pragma unroll
@@ -411,6 +439,8 @@ inline int phase_probe() {
         if (run_phase<2, 2>("reference as a fifth k-step, no fma", blocks, out, clk, data)) return 2;
         if (run_phase<3, 2>("row sums by v_add_f32", blocks, out, clk, data)) return 2;
         if (run_phase<4, 2>("half the row-sum mfma, pk_add_f16", blocks, out, clk, data)) return 2;
+        if (run_phase<5, 2>("products as 16x16x32 tiles", blocks, out, clk, data)) return 2;
+        if (run_phase<5, 1>("products as 16x16x32 tiles", blocks, out, clk, data)) return 2;
     }
     (void)hipFree(out);
     (void)hipFree(clk);

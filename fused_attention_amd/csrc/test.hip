@@ -59,6 +59,28 @@ __global__ __launch_bounds__(512) void mfma_peak_kernel(float* out, const half8*
     out[blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// The same flops through v_mfma_f32_16x16x32_f16 (half the flops per instruction, a quarter of the
+// accumulator registers): does the other tile shape of the matrix core sustain more on real data?
+__global__ __launch_bounds__(512) void mfma_peak_kernel_16(float* out, const half8* data, int iters) {
+    typedef float floatx4 __attribute__((ext_vector_type(4)));
+    half8 a[4], b[4];
+    for (int i = 0; i < 4; i++) {
+        a[i] = data[threadIdx.x + i * 512];
+        b[i] = data[threadIdx.x + (i + 4) * 512];
+    }
+    floatx4 c[8];
+    for (int n = 0; n < 8; n++) c[n] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int j = 0; j < 32; j++)
+            c[j % 8] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j % 4], b[(j / 4) % 4], c[j % 8], 0, 0, 0);
+    }
+    float s = 0.f;
+    for (int n = 0; n < 8; n++)
+        for (int r = 0; r < 4; r++) s += c[n][r];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 int mfma_peak() {
     hipDeviceProp_t prop;
     HIP_OK(hipGetDeviceProperties(&prop, 0));
@@ -84,21 +106,24 @@ int mfma_peak() {
     hipEvent_t e0, e1;
     HIP_OK(hipEventCreate(&e0));
     HIP_OK(hipEventCreate(&e1));
-    for (int rep = 0; rep < 2; ++rep) {
+    for (int rep = 0; rep < 4; ++rep) {
+        // passes 0 and 1: 32x32x16; passes 2 and 3: 16x16x32 (the same flops per loop iteration)
+        auto kernel = rep < 2 ? mfma_peak_kernel : mfma_peak_kernel_16;
         for (int kind = 0; kind < 2; ++kind) {
             const half8* d = kind == 0 ? dz : dn;
-            hipLaunchKernelGGL(mfma_peak_kernel, dim3(blocks), dim3(threads), 0, nullptr, out, d, 200);
+            hipLaunchKernelGGL(kernel, dim3(blocks), dim3(threads), 0, nullptr, out, d, 200);
             HIP_OK(hipEventRecord(e0, nullptr));
             for (int r = 0; r < 3; ++r)
-                hipLaunchKernelGGL(mfma_peak_kernel, dim3(blocks), dim3(threads), 0, nullptr, out, d, iters);
+                hipLaunchKernelGGL(kernel, dim3(blocks), dim3(threads), 0, nullptr, out, d, iters);
             HIP_OK(hipEventRecord(e1, nullptr));
             HIP_OK(hipEventSynchronize(e1));
             float ms = 0.f;
             HIP_OK(hipEventElapsedTime(&ms, e0, e1));
             ms /= 3.f;
             const double flop = (double)blocks * (threads / 64) * iters * 16.0 * 32768.0;
-            std::printf("mfma-peak %-16s %d CUs x 8 waves: %.3f ms per launch, %.0f TFLOP/s\n",
-                        kind == 0 ? "zero operands" : "N(0,1) operands", blocks, ms, flop / ms / 1e9);
+            std::printf("mfma-peak %s %-16s %d CUs x 8 waves: %.3f ms per launch, %.0f TFLOP/s\n",
+                        rep < 2 ? "32x32x16" : "16x16x32", kind == 0 ? "zero operands" : "N(0,1) operands", blocks, ms,
+                        flop / ms / 1e9);
         }
     }
     (void)hipFree(dz);
