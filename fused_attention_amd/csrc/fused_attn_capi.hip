@@ -108,8 +108,8 @@ Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask, bool
             if (1024.0 * useful / held * rows_used >= 614.0) return H > 64 ? Shape{8, 1} : Shape{8, 2};
         }
     }
-    // (With a mask a lone round may be emptier still: the four-wave alternative is slower there.)
-    const bool pingpong = wgs8 >= 2 * kNumCu ? usage8 >= 614 : usage8 >= (wgs8 <= kNumCu ? (has_mask ? 560 : 614) : 717);
+    // Usage of 0.55 in a lone round, 0.7 in a part-filled second round, 0.6 from two rounds on.
+    const bool pingpong = wgs8 >= 2 * kNumCu ? usage8 >= 614 : usage8 >= (wgs8 <= kNumCu ? 560 : 717);
     // 256-query workgroups with an additive mask: up to 30 % faster than the four-wave kernel,
     // whose masked loop is not pipelined, from 160 workgroups on, unless a quarter or more of the
     // query rows of a head's workgroups do not exist.
@@ -119,10 +119,10 @@ Shape pick_shape(int64_t B, int64_t R, int64_t L, int64_t H, bool has_mask, bool
     if (pingpong) return {8, 2};
     // 256-query ping-pong workgroups.  Thresholds from sweeps of mid-size shapes on MI355X.
     // Causal (a workgroup takes a pair of 256-query tiles, one resident per compute unit): 4 to
-    // 21 % faster than the four-wave kernel when the pairs fill 60 % or more of a single round,
+    // 21 % faster than the four-wave kernel when the pairs fill 55 % or more of a single round,
     // slower on emptier or on several rounds.
     if (causal)
-        return heads * ceil_div(L, 512) <= kNumCu && usage(heads, L, 512, kNumCu) >= 614 ? Shape{8, 1} : Shape{4, 1};
+        return heads * ceil_div(L, 512) <= kNumCu && usage(heads, L, 512, kNumCu) >= 560 ? Shape{8, 1} : Shape{4, 1};
     // Additive mask: one resident per compute unit.
     if (has_mask) return masked81 ? Shape{8, 1} : Shape{4, 1};
     // Plain, two per compute unit: per compute unit they run at 0.93 of the 512-query ones and
