@@ -22,11 +22,23 @@ if REPO not in sys.path:
 
 PEAK_TFLOPS_FP16 = 2500.0   # MI355X dense fp16 MFMA, published
 
-# HBM bytes per launch of the forward kernel, measured with rocprofv3 (FETCH_SIZE and WRITE_SIZE
-# in separate --pmc runs of this script, each scaled by what the same counter reads for the 1 GiB
-# calibration copy below: 2.000 for fetch, 1.000 for write).  Summaries:
-# profiles/fwd_kernel_pingpong_c3.md and profiles/fwd_kernel_pingpong_c4.md.
-MEASURED_TRAFFIC_BYTES = {"c3": 134.4e6, "c4": 808.2e6}
+# HBM bytes per launch of the forward kernel.  They are not measured by this script: they were read
+# with rocprofv3 (FETCH_SIZE and WRITE_SIZE in separate --pmc runs of this script, each scaled by
+# what the same counter reads for the 1 GiB calibration copy below: 2.000 for fetch, 1.000 for
+# write) and are quoted here with the file that holds the counter summary.  Workloads without a
+# counter run report null.
+MEASURED_TRAFFIC = {
+    "c3": (134.4e6, "profiles/fwd_kernel_pingpong_c3.md"),
+    "c4": (808.2e6, "profiles/fwd_kernel_pingpong_c4.md"),
+}
+
+# Launches made before the counted warm-up until this much time has passed: the chip needs a few
+# hundred milliseconds of work before its clock settles (a 25-launch run reads about 10 % low).
+SETTLE_SECONDS = 0.5
+
+# The other benchmark configurations, measured after the headline line's timed region: seconds of
+# event-timed launches per workload, and host seconds for the error check of each.
+OTHER_WORKLOADS = ("c1", "c2", "c4", "c5a", "c5b", "readme")
 
 
 def cpu_baseline(w, q, k, v, gpu_out, budget_s):
@@ -65,6 +77,68 @@ def cpu_baseline(w, q, k, v, gpu_out, budget_s):
     }
 
 
+def settle(step, seconds):
+    """Launches `step` until `seconds` have passed; returns the number of launches."""
+    import torch
+
+    n = 0
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            step()
+        torch.cuda.synchronize()
+        n += 8
+    return n
+
+
+def side_workload(name, dev, check_budget_s):
+    """Kernel time, TFLOP/s and error on a bounded sample of (batch, head) pairs for one of the
+    configurations that are not the headline: HIP events around back-to-back launches inside the
+    kernel library, after a settle loop of its own."""
+    import torch
+
+    import fused_attn
+    from fused_attention_amd import capi, workloads
+    from oracle import attention_per_head
+
+    w = workloads.WORKLOADS[name]
+    q, k, v = workloads.make_inputs(w)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    out = fused_attn.attention_forward(w.H, min(128, 2 * w.H), qd, kd, vd)
+    torch.cuda.synchronize()
+    one = max(capi.forward_timed(qd, kd, vd, w.H, out, iters=3), 1e-3)
+    settle_iters = max(8, int(0.3e3 / one))
+    capi.forward_timed(qd, kd, vd, w.H, out, iters=settle_iters)
+    iters = max(50, min(5000, int(0.3e3 / one)))
+    kernel_ms = capi.forward_timed(qd, kd, vd, w.H, out, iters=iters)
+    flop = workloads.flops(w)
+    tflops = flop / (kernel_ms * 1e-3) / 1e12
+    entry = {
+        "shape": "B=%d R=%d L=%d H=%d" % (w.B, w.R, w.L, w.H),
+        "kernel_ms": kernel_ms,
+        "launches_timed": iters,
+        "tflops": tflops,
+        "frac": tflops / PEAK_TFLOPS_FP16,
+    }
+    if check_budget_s > 0:
+        pairs_all = [(b, h) for b in range(w.B) for h in range(w.R)]
+        t0 = time.perf_counter()
+        ref = attention_per_head(q, k, v, w.H, heads=pairs_all[:1])
+        per_pair = time.perf_counter() - t0
+        n = max(1, min(len(pairs_all), int(check_budget_s / max(per_pair, 1e-6))))
+        # spread over batches and heads; the first pair has been computed already
+        extra = pairs_all[1::max(1, len(pairs_all) // n)][:n - 1]
+        if extra:
+            more = attention_per_head(q, k, v, w.H, heads=extra)
+            ref = torch.where(torch.isnan(ref), more, ref)
+        got = out.float().cpu()
+        sel = ~torch.isnan(ref)
+        entry["max_abs_err"] = (got[sel] - ref[sel]).abs().max().item()
+        entry["finite"] = bool(torch.isfinite(got).all())
+        entry["pairs_checked"] = 1 + len(extra)
+    return entry
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -78,6 +152,11 @@ def main():
                     help="size of the plain copy run before the timed region (0 disables it)")
     ap.add_argument("--cpu-budget-s", type=float, default=15.0,
                     help="seconds of host time for the CPU baseline sample (0 disables it)")
+    ap.add_argument("--others", choices=["auto", "on", "off"], default="auto",
+                    help="also measure the other benchmark configurations into \"workloads\" "
+                         "(auto: with the default headline workload, non-causal)")
+    ap.add_argument("--check-budget-s", type=float, default=4.0,
+                    help="host seconds per workload for the error check of the other configurations")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the forward has no multi-GPU path "
@@ -116,6 +195,7 @@ def main():
         def step():
             return fused_attn.attention_forward(w.H, chunk, qd, kd, vd)
 
+    settle_launches = settle(step, SETTLE_SECONDS)
     for _ in range(args.warmup):
         out = step()
     torch.cuda.synchronize()
@@ -150,6 +230,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_launches": settle_launches,
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
@@ -169,12 +250,19 @@ def main():
             "peak": PEAK_TFLOPS_FP16,
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_TFLOPS_FP16,
-            "traffic": None if args.causal else MEASURED_TRAFFIC_BYTES.get(w.name),
+            "traffic": None if args.causal else MEASURED_TRAFFIC.get(w.name, (None, None))[0],
+            "traffic_source": None if args.causal else MEASURED_TRAFFIC.get(w.name, (None, None))[1],
             "kernel_ms": kernel_ms,
         },
     }
     if args.cpu_budget_s > 0 and not args.causal:
         line["cpu_baseline"] = cpu_baseline(w, q, k, v, out, args.cpu_budget_s)
+    others = args.others == "on" or (args.others == "auto" and args.workload == "c3" and not args.causal)
+    if others:
+        del qd, kd, vd, out
+        torch.cuda.empty_cache()
+        line["workloads"] = {name: side_workload(name, dev, args.check_budget_s)
+                             for name in OTHER_WORKLOADS if name != args.workload}
     print(json.dumps(line))
 
 

@@ -1,7 +1,8 @@
 """ctypes view of libfused_attn_gfx950.so (the C ABI declared in include/fused_attn.h).
 
-The functions here only marshal pointers, sizes and strides; all checking of those values is
-done by the library and reported through its status codes.
+`forward` and `forward_timed` check what the library cannot see from raw addresses (tensor
+devices, shapes, the mask's extent) and raise before any address reaches it; value ranges,
+alignment and strides are checked by the library and reported through its status codes.
 """
 import ctypes
 import math
@@ -108,6 +109,62 @@ def _current_stream(q):
     return torch.cuda.current_stream(q.device).cuda_stream
 
 
+def _checked_problem(q, k, v, head_dim, out, mask, layout):
+    """Everything the library cannot see from raw addresses, checked before any address reaches it
+    (the same checks as the torch binding, reference src/fused_attn_extention.cu:24-64): dtypes,
+    GPU residency on one device, dimensionality, equal shapes and strides, num_features a
+    multiple of head_dim, a contiguous [B, L, L] mask.  Returns (B, R, L, q/k/v strides).
+    Raises TypeError / ValueError; needs neither the library nor a GPU to do so."""
+    import torch
+
+    named = (("q", q), ("k", k), ("v", v), ("out", out), ("mask", mask))
+    for name, t in named:
+        if t is not None and not isinstance(t, torch.Tensor):
+            raise TypeError("%s must be a torch.Tensor, got %s" % (name, type(t).__name__))
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("q, k, v must be float16 or bfloat16, got %s" % q.dtype)
+    for name, t in named[1:]:
+        if t is not None and t.dtype != q.dtype:
+            raise TypeError("%s must have the dtype of q (%s), got %s" % (name, q.dtype, t.dtype))
+    if int(head_dim) != head_dim or head_dim not in (16, 32, 64, 128):
+        raise ValueError("head_dim must be 16, 32, 64 or 128, got %r" % (head_dim,))
+    if layout not in ("blf", "bhld"):
+        raise ValueError("layout must be 'blf' or 'bhld'")
+    want_dim = 3 if layout == "blf" else 4
+    if q.dim() != want_dim:
+        raise ValueError("layout %r takes %d-D tensors, q has %d dimensions" % (layout, want_dim, q.dim()))
+    if layout == "blf":
+        if q.shape[2] % head_dim != 0:
+            raise ValueError("num_features (%d) must be a multiple of head_dim (%d)" % (q.shape[2], head_dim))
+    elif q.shape[3] != head_dim:
+        raise ValueError("the last dimension (%d) must equal head_dim (%d)" % (q.shape[3], head_dim))
+    if min(q.shape) < 1:
+        raise ValueError("q must not have an empty dimension, got %s" % (tuple(q.shape),))
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("q, k, v must have one shape")
+    if out is not None and out.shape != q.shape:
+        raise ValueError("out must have the shape of q")
+    B, R, L = _layout(q, head_dim, layout)[:3]
+    strides = _strides(q, head_dim, layout, "q")
+    if _strides(k, head_dim, layout, "k") != strides or _strides(v, head_dim, layout, "v") != strides:
+        raise ValueError("q, k, v must have the same strides")
+    if mask is not None:
+        if tuple(mask.shape) != (B, L, L):
+            raise ValueError("mask must have shape [batch, seq_len, seq_len] = [%d, %d, %d], got %s"
+                             % (B, L, L, tuple(mask.shape)))
+        if not mask.is_contiguous():
+            raise ValueError("mask must be contiguous")
+    # last, so that the checks above can be exercised on host tensors
+    for name, t in named:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("%s must be a GPU tensor, got device %s" % (name, t.device))
+        if t.device != q.device:
+            raise ValueError("%s is on %s but q is on %s" % (name, t.device, q.device))
+    return B, R, L, strides
+
+
 def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None, causal=False,
             return_lse=False):
     """Runs fa_fwd_strided on torch GPU tensors (fp16 or bf16) on torch's current stream.
@@ -115,30 +172,17 @@ def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None, ca
     layout 'blf' takes [B, L, R*head_dim] tensors, 'bhld' takes [B, R, L, head_dim] tensors.
     q, k and v may be views (slices of one packed projection output, say) as long as their last
     dimension is dense and the three have the same strides; `out` may be a view of its own.  The
-    mask is contiguous [B, L, L].  causal=True restricts query i to keys j <= i.  q, k, v (and out, mask when given) must share
-    one dtype; bfloat16 tensors set FA_FLAG_BF16.  Returns `out` (allocated like q when not
-    given), or (out, lse) with lse a float32 [B, R, L] tensor when return_lse is set.
+    mask is contiguous [B, L, L].  causal=True restricts query i to keys j <= i.  q, k, v (and out,
+    mask when given) must share one dtype and one GPU; bfloat16 tensors set FA_FLAG_BF16.  Returns
+    `out` (allocated like q when not given), or (out, lse) with lse a float32 [B, R, L] tensor
+    when return_lse is set.
     """
     import torch
 
-    if q.dtype not in (torch.float16, torch.bfloat16):
-        raise TypeError("q, k, v must be float16 or bfloat16, got %s" % q.dtype)
-    for name, t in (("k", k), ("v", v), ("out", out), ("mask", mask)):
-        if t is not None and t.dtype != q.dtype:
-            raise TypeError("%s must have the dtype of q (%s), got %s" % (name, q.dtype, t.dtype))
+    B, R, L, (sb, sh, sl) = _checked_problem(q, k, v, head_dim, out, mask, layout)
     flags = (FLAG_CAUSAL if causal else 0) | (FLAG_BF16 if q.dtype == torch.bfloat16 else 0)
-    B, R, L = _layout(q, head_dim, layout)[:3]
-    if k.shape != q.shape or v.shape != q.shape:
-        raise ValueError("q, k, v must have one shape")
-    sb, sh, sl = _strides(q, head_dim, layout, "q")
-    if _strides(k, head_dim, layout, "k") != (sb, sh, sl) or _strides(v, head_dim, layout, "v") != (sb, sh, sl):
-        raise ValueError("q, k, v must have the same strides")
-    if mask is not None and not mask.is_contiguous():
-        raise ValueError("mask must be contiguous")
     if out is None:
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    elif out.shape != q.shape:
-        raise ValueError("out must have the shape of q")
     ob, oh, ol = _strides(out, head_dim, layout, "out")
     if scale is None:
         scale = 1.0 / math.sqrt(head_dim)
@@ -154,10 +198,15 @@ def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None, ca
 
 def forward_timed(q, k, v, head_dim, out, iters, mask=None, layout="blf", scale=None):
     """Average milliseconds per launch over `iters` back-to-back launches (HIP events on the
-    launch stream, measured inside the library)."""
+    launch stream, measured inside the library).  fp16 only; q, k, v and out share one set of
+    strides (fa_fwd_timed has no output strides of its own)."""
     import torch
 
-    B, R, L, sb, sh, sl = _layout(q, head_dim, layout)
+    B, R, L, (sb, sh, sl) = _checked_problem(q, k, v, head_dim, out, mask, layout)
+    if q.dtype != torch.float16:
+        raise TypeError("forward_timed takes float16 tensors, got %s" % q.dtype)
+    if out is None or _strides(out, head_dim, layout, "out") != (sb, sh, sl):
+        raise ValueError("forward_timed needs an `out` tensor with the strides of q")
     if scale is None:
         scale = 1.0 / math.sqrt(head_dim)
     ms = ctypes.c_float(0.0)

@@ -60,7 +60,27 @@ struct CausalPlan {
     int64_t blocks;       // key blocks the busiest workgroup walks through
 };
 
+CausalPlan plan_causal_walk(int64_t heads, int64_t n, int64_t H);
+
+// One causal launch asks for its plan twice (shape choice, then grid), and a serving loop asks for
+// the same few plans over and over: the last results are kept per host thread.
 CausalPlan plan_causal(int64_t heads, int64_t n, int64_t H) {
+    struct Entry {
+        int64_t heads, n, H;
+        CausalPlan plan;
+    };
+    constexpr int kEntries = 8;
+    thread_local Entry cache[kEntries] = {};
+    thread_local int next = 0;
+    for (const Entry& e : cache)
+        if (e.heads == heads && e.n == n && e.H == H) return e.plan;
+    const CausalPlan plan = plan_causal_walk(heads, n, H);
+    cache[next] = Entry{heads, n, H, plan};
+    next = (next + 1) % kEntries;
+    return plan;
+}
+
+CausalPlan plan_causal_walk(int64_t heads, int64_t n, int64_t H) {
     const int64_t pairs = heads * ceil_div(n, 2);
     const CausalPlan paired{false, ceil_div(pairs, kNumCu) * (n + 1)};
     constexpr int kPerXcd = kNumCu / fa::kNumXcd;
@@ -157,8 +177,10 @@ hipError_t launch(const fa::FwdParams& p, hipStream_t stream) {
         if (e != hipSuccess) return e;
     }
     const int grid = p.wgs_per_xcd * fa::kNumXcd;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * 64), lds, stream, p);
-    return hipGetLastError();
+    // the launch's own status, not the thread's sticky last error (which may stem from the caller's code)
+    fa::FwdParams params = p;
+    void* args[] = {&params};
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(NW * 64), args, lds, stream);
 }
 
 template <int H, int NW, int NQB, int WPE, int MODE, bool BF>
@@ -170,8 +192,10 @@ hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
         if (e != hipSuccess) return e;
     }
     const int grid = p.wgs_per_xcd * fa::kNumXcd;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * 64), lds, stream, p);
-    return hipGetLastError();
+    // the launch's own status, not the thread's sticky last error (which may stem from the caller's code)
+    fa::FwdParams params = p;
+    void* args[] = {&params};
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(NW * 64), args, lds, stream);
 }
 
 template <int H, int MODE, bool BF>

@@ -200,9 +200,16 @@ struct TileLoader {
 // Largest partial row sum (16 terms) the fast path of the online softmax accepts.
 constexpr float kTrip = 16384.f;
 
-// Eight-wave kernel: bias (log2 units) of the reference the exponentials are taken against, and the
-// largest sum of a query's 32 probabilities of one sub-tile that its fast path accepts.
-constexpr float kBias = 6.0f;
+// Bias (log2 units) of the reference the exponentials are taken against, in every kernel, and the
+// largest sum of a query's 32 probabilities of one sub-tile that the eight-wave kernel's fast path
+// accepts.  The bias
+// is negative: a key at the reference maximum gets the probability 2^-kBias = 16, so that the
+// fp16 rounding of the probabilities (normal numbers down to 2^-14, subnormals down to 2^-24)
+// reaches 28 log2 units below the maximum before a weight is lost: a tail of L small weights
+// then loses at most L 2^-28 of the row (2.4e-4 at L = 65536).  The reference may lag the true
+// maximum by 15 + kBias = 11 log2 units (10 in the four-wave kernels, whose check works on half
+// rows) before the check sends the wave down the slow path.
+constexpr float kBias = -4.0f;
 constexpr float kTripSum = 32768.f;
 
 // O^T[.][nb] *= alpha, in place.  Written as one instruction per register with the register tied

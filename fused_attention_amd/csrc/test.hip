@@ -8,8 +8,6 @@
 // usage: fa_test [B R L H [iters [blhd|bhld [input_scale [qzero|vconst|vcol]]]]]
 //        fa_test mfma-peak        what v_mfma_f32_32x32x16_f16 sustains on this chip with zero
 //                                 operands and with N(0,1) operands (the rate depends on the data)
-//        fa_test issue-probe      how matrix and vector instructions of the waves of one SIMD overlap
-//        fa_test phase-probe      the compute of the eight-wave kernel without its memory traffic, on all CUs
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -20,7 +18,6 @@
 #include <vector>
 
 #include "../../include/fused_attn.h"
-#include "issue_probe.hpp"
 
 #define HIP_OK(expr)                                                                          \
     do {                                                                                      \
@@ -149,8 +146,6 @@ int main(int argc, char** argv) {
     bool bhld = false;
     float amp = 1.7320508f;  // uniform with unit variance
     if (argc >= 2 && std::strcmp(argv[1], "mfma-peak") == 0) return mfma_peak();
-    if (argc >= 2 && std::strcmp(argv[1], "issue-probe") == 0) return probe::issue_probe();
-    if (argc >= 2 && std::strcmp(argv[1], "phase-probe") == 0) return probe::phase_probe();
     if (argc >= 5) {
         B = std::atoll(argv[1]);
         R = std::atoll(argv[2]);

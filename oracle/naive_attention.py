@@ -78,12 +78,14 @@ def causal_mask(batch_size, sequence_len):
     return m.expand(batch_size, sequence_len, sequence_len).contiguous()
 
 
-def attention_per_head(queries, keys, values, head_dim, heads=None):
+def attention_per_head(queries, keys, values, head_dim, heads=None, rows=None):
     """Same arithmetic as `attention`, one (batch, head) at a time.
 
     The one-shot form materialises two float32 [B, R, L, L] tensors (2 x 4 GiB at B=4, R=16,
     L=4096; 2 x 32 GiB at R=32, L=16384).  This form needs 2 x 4 L^2 bytes at a time.
     heads: optional iterable of (batch, head) pairs to evaluate; the others are left as NaN.
+    rows: optional 1-D index tensor of query positions to evaluate (all keys are always used);
+    the other rows are left as NaN.  Pinned against `attention` in tests/test_oracle.py.
     """
     batch_size, sequence_len, num_features = queries.shape
     num_heads = num_features // head_dim
@@ -95,8 +97,13 @@ def attention_per_head(queries, keys, values, head_dim, heads=None):
         q = queries[b, :, cols].to(torch.float32)
         k = keys[b, :, cols].to(torch.float32)
         v = values[b, :, cols].to(torch.float32)
+        if rows is not None:
+            q = q[rows]
         scores = torch.softmax((q @ k.mT) * inv, dim=-1)
-        out[b, :, cols] = scores @ v
+        if rows is not None:
+            out[b, rows, cols] = scores @ v
+        else:
+            out[b, :, cols] = scores @ v
     return out
 
 

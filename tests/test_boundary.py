@@ -197,3 +197,44 @@ def test_python_wrapper_forwards_to_the_binding():
 
     sig = inspect.signature(fused_attention_amd.attention_forward)
     assert list(sig.parameters) == ["head_dim", "chunk_size", "queries", "keys", "values", "mask"]
+
+
+def test_ctypes_wrapper_checks_tensors_before_any_address_reaches_the_library(monkeypatch):
+    # The library sees raw addresses only: a host tensor, a mask of the wrong extent or a feature
+    # count that head_dim does not divide must raise here, not fault on the GPU (the same checks
+    # as the binding's, reference src/fused_attn_extention.cu:24-64).
+    def no_library():
+        raise AssertionError("the library was reached")
+
+    monkeypatch.setattr(capi, "load_library", no_library)
+    B, L, R, H = 2, 64, 2, 64
+    q = torch.zeros(B, L, R * H, dtype=torch.float16)
+    out = torch.zeros_like(q)
+
+    def both(match, exc=ValueError, **kw):
+        args = dict(q=q, k=q, v=q, head_dim=H, out=out)
+        args.update(kw)
+        with pytest.raises(exc, match=match):
+            capi.forward(**args)
+        with pytest.raises(exc, match=match):
+            capi.forward_timed(iters=1, **args)
+
+    both("GPU tensor")                                              # host tensors, everything else in order
+    for bad_mask in (torch.zeros(1, L, L), torch.zeros(L, L), torch.zeros(B, 1, L, L), torch.zeros(B, L, L - 8),
+                     torch.zeros(B, L + 8, L + 8)):
+        both("mask must have shape", mask=bad_mask.half())
+    both("mask must be contiguous", mask=torch.zeros(B, L, 2 * L, dtype=torch.float16)[:, :, ::2])
+    both("dtype of q", exc=TypeError, mask=torch.zeros(B, L, L))
+    both("multiple of head_dim", head_dim=128, q=q[:, :, :H + 32], k=q[:, :, :H + 32], v=q[:, :, :H + 32],
+         out=out[:, :, :H + 32])
+    both("head_dim must be", head_dim=48)
+    both("one shape", k=q[:, :32])
+    both("same strides", k=torch.zeros(B, L, 2 * R * H, dtype=torch.float16)[:, :, :R * H])
+    both("3-D", q=q[0], k=q[0], v=q[0], out=out[0])
+    both("4-D", layout="bhld")
+    both("last dimension", layout="bhld", q=q.view(B, L, R, H), k=q.view(B, L, R, H), v=q.view(B, L, R, H),
+         out=out.view(B, L, R, H), head_dim=32)
+    both("float16 or bfloat16", exc=TypeError, q=q.float(), k=q.float(), v=q.float(), out=out.float())
+    both("torch.Tensor", exc=TypeError, k=[1, 2, 3])
+    with pytest.raises(ValueError, match="shape of q"):
+        capi.forward(q, q, q, H, out=out[:, :32])

@@ -56,6 +56,29 @@ def test_simple(gpu, head_dim, chunk_size):
     assert _max_err(actual, expected) <= TOL
 
 
+def test_reference_test_body_through_the_shim(gpu):
+    # The body of the reference's run_simple_test (reference tests/test_fused_attn.py:12-30) with
+    # its own imports: `import fused_attn`, `from naive_implementation import attention`, and
+    # assert_close on the two fp16 tensors as they come.
+    import os
+    import sys
+
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    try:
+        from naive_implementation import attention as shim_attention
+    finally:
+        sys.path.pop(0)
+    import fused_attn
+
+    head_dim, chunk_size = 64, 64
+    torch.random.manual_seed(179)
+    queries, keys, values = (torch.randn(1, 2 * chunk_size, 2 * head_dim).half().to(gpu) for _ in range(3))
+    expected = shim_attention(queries.cpu(), keys.cpu(), values.cpu(), head_dim)
+    actual = fused_attn.attention_forward(head_dim, chunk_size, queries, keys, values)
+    assert expected.dtype == actual.dtype == torch.float16
+    torch.testing.assert_close(actual.cpu(), expected, rtol=0.01, atol=0.01)
+
+
 # ---- benchmark configurations -------------------------------------------------------------------
 
 @pytest.mark.parametrize("name", ["c1", "c2", "c5a", "c5b"])
@@ -90,17 +113,67 @@ def test_config_c3_headline(gpu):
     assert (got.view(w.B, w.L, w.R, w.H).abs() <= vmax + 1e-3).all()
 
 
+def _sample_rows(L, n, seed):
+    """Query positions to check: the first and last rows of the sequence (first and last query
+    tiles, wave boundaries) and a seeded sample of the rest."""
+    g = torch.Generator().manual_seed(seed)
+    edge = torch.cat([torch.arange(0, min(L, 96)), torch.arange(max(0, L - 96), L)])
+    rand = torch.randperm(L, generator=g)[:n]
+    return torch.unique(torch.cat([edge, rand]))
+
+
+def _check_whole_tensor_without_an_oracle(forward, q, k, v, w, got, gpu):
+    """Two checks that touch every (batch, head, row): a convex combination stays inside the range
+    of the head's values, and zero queries return the mean of the head's values."""
+    vh = v.float().view(w.B, w.L, w.R, w.H)
+    vmax = vh.abs().amax(dim=1, keepdim=True).expand(w.B, w.L, w.R, w.H)
+    assert (got.view(w.B, w.L, w.R, w.H).abs() <= vmax + 1e-3).all()
+    flat = forward(torch.zeros_like(q).to(gpu), k.to(gpu), v.to(gpu)).float().cpu()
+    mean = vh.mean(dim=1, keepdim=True).expand(w.B, w.L, w.R, w.H)
+    assert (flat.view(w.B, w.L, w.R, w.H) - mean).abs().max().item() <= 2e-3
+
+
 def test_config_c4_sampled_heads(gpu):
     import fused_attn
 
     w = workloads.WORKLOADS["c4"]
     q, k, v = workloads.make_inputs(w)
-    got = fused_attn.attention_forward(w.H, 128, q.to(gpu), k.to(gpu), v.to(gpu)).float().cpu()
+
+    def forward(q, k, v):
+        return fused_attn.attention_forward(w.H, 128, q, k, v)
+
+    got = forward(q.to(gpu), k.to(gpu), v.to(gpu)).float().cpu()
     assert torch.isfinite(got).all()
-    pairs = [(0, 0), (0, 13), (0, 31)]       # first, middle and last head; all 16384 rows of each
+    # Eight heads, one per residue modulo 8 (the kernel renumbers workgroups per XCD, so a mistake
+    # there would depend on the head): ~2200 rows of each, every key.
+    pairs = [(0, h) for h in (0, 5, 10, 15, 16, 21, 26, 31)]
+    rows = _sample_rows(w.L, 2048, 4)
+    want = attention_per_head(q, k, v, w.H, heads=pairs, rows=rows)
+    sel = ~torch.isnan(want)
+    assert sel.sum().item() == len(pairs) * rows.numel() * w.H
+    assert (got[sel] - want[sel]).abs().max().item() <= TOL
+    _check_whole_tensor_without_an_oracle(forward, q, k, v, w, got, gpu)
+
+
+def test_config_reference_benchmark_shape(gpu):
+    # The shape of the reference's own benchmark (reference tests/benchmark_fused_attn.py:9-15:
+    # batch 4, 40 heads, sequence 2048, head_dim 128, chunk 128), which the reference times but
+    # never checks.
+    import fused_attn
+
+    w = workloads.WORKLOADS["readme"]
+    q, k, v = workloads.make_inputs(w)
+
+    def forward(q, k, v):
+        return fused_attn.attention_forward(w.H, 128, q, k, v)
+
+    got = forward(q.to(gpu), k.to(gpu), v.to(gpu)).float().cpu()
+    assert torch.isfinite(got).all()
+    pairs = [(b, h) for b in range(w.B) for h in range(w.R) if (b * w.R + h) % 9 == 0]   # 18 of 160, every residue mod 8
     want = attention_per_head(q, k, v, w.H, heads=pairs)
     sel = ~torch.isnan(want)
     assert (got[sel] - want[sel]).abs().max().item() <= TOL
+    _check_whole_tensor_without_an_oracle(forward, q, k, v, w, got, gpu)
 
 
 def test_full_size_properties_without_an_oracle(gpu):
@@ -690,6 +763,30 @@ def test_eight_wave_kernel_reference_lag(gpu, B, R, L, H, step_log2):
     if step_log2 >= 14:
         want = v[:, 96:].float().mean(dim=1, keepdim=True)
         assert (got.float().cpu() - want).abs().max().item() <= 5e-3
+
+
+@pytest.mark.parametrize("B,R,L,H", [(2, 16, 4096, 64), (1, 8, 16384, 128), (1, 2, 1024, 64)])
+@pytest.mark.parametrize("gap_log2", [10.5, 14.5, 16.5, 17.5, 18.5, 19.0, 22.0])
+def test_heavy_tail_of_small_weights(gpu, B, R, L, H, gap_log2):
+    # One dominant key, then L - 1 equal keys gap_log2 (log2 units) below it.  Each of them weighs
+    # 2^-gap, together (L - 1) 2^-gap: 6 % of the row at gap 18 and L = 16384.  The probabilities
+    # are rounded to fp16 before the second product, so a kernel whose reference pushes such
+    # weights into the fp16 subnormals (or below 2^-24, to zero) loses that share of the row; the
+    # float32 oracle keeps it.  Both kernel families, through eight-wave and four-wave grids.
+    t = gap_log2 / math.log2(math.e) / math.sqrt(H)      # key 0 = t * ones: scaled score H t / sqrt(H)
+    q = torch.ones(B, L, R * H).half()
+    k = torch.zeros(B, L, R * H)
+    k[:, 0] = t
+    k = k.half()
+    gap = k[0, 0, 0].float().item() * math.sqrt(H) * math.log2(math.e)      # what fp16 made of it
+    v = _rand((B, L, R * H), 4400 + L)
+    v[:, 0] = 4.0                                      # the dominant key's value stands out
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H)
+    assert torch.isfinite(got.float()).all()
+    tail = (L - 1) * 2.0 ** -gap
+    want = (4.0 + tail * v[:, 1:].float().mean(dim=1)) / (1.0 + tail)       # closed form, every row the same
+    assert (got.float().cpu() - want.view(B, 1, R * H)).abs().max().item() <= TOL
+    _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R - 1)])
 
 
 @pytest.mark.parametrize("B,R,L,H", [

@@ -76,6 +76,11 @@ def test_per_head_form_is_the_same_arithmetic():
     part = attention_per_head(q, k, v, H, heads=[(1, 2)])
     assert torch.isnan(part[0]).all() and torch.isnan(part[1, :, : 2 * H]).all()
     torch.testing.assert_close(part[1, :, 2 * H:], attention(q, k, v, H)[1, :, 2 * H:], rtol=0, atol=1e-6)
+    # a subset of the query rows: the same rows of the full answer, the others untouched
+    rows = torch.tensor([0, 7, 64, 149])
+    some = attention_per_head(q, k, v, H, heads=[(0, 1)], rows=rows)
+    torch.testing.assert_close(some[0, rows, H:2 * H], attention(q, k, v, H)[0, rows, H:2 * H], rtol=0, atol=1e-6)
+    assert torch.isnan(some).sum().item() == some.numel() - rows.numel() * H
 
 
 def test_head_h_is_columns_hH_to_hH_plus_H():
@@ -193,3 +198,49 @@ def test_causal_mask_means_prefix_attention():
     for i in (0, 1, 7, L - 1):
         prefix = attention(*(t[:, :i + 1].contiguous() for t in (q, k, v)), H)
         torch.testing.assert_close(causal[:, i], prefix[:, i], rtol=0, atol=2e-6)
+
+
+# ---- the rounding model of the kernels' probabilities, on the host ------------------------------
+
+def _rtz_fp16(x):
+    """float32 -> fp16 rounded toward zero (what v_cvt_pkrtz_f16_f32 does), for x >= 0."""
+    h = x.to(torch.float16)
+    up = h.float() > x
+    bits = h.view(torch.int16) - up.to(torch.int16)
+    return bits.view(torch.float16)
+
+
+def _kernel_bias_log2():
+    import os
+    import re
+
+    here = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(here, "fused_attention_amd", "csrc", "fused_attn_kernel.hpp")).read()
+    return float(re.search(r"constexpr float kBias = (-?[0-9.]+)f;", text).group(1))
+
+
+def test_rounding_model_of_small_weights():
+    # The eight-wave kernel rounds p = exp2(score - reference - bias) toward zero to fp16 before
+    # the second product.  fp16 has normal numbers down to 2^-14 and subnormals down to 2^-24, so
+    # keys more than 24 - bias log2 units below the reference vanish and keys in the ten units
+    # above that are truncated.  Worst case over the gap: one dominant key and L - 1 keys `gap`
+    # below it; the lost share of the row is at most (L - 1) 2^-(24 - bias).  With the bias the
+    # kernel header states, that stays inside half the 5e-3 bound up to L = 65536 for values of
+    # magnitude 4; a bias of +6 (reference 64 times above the maximum) would not.
+    def worst_error(L, bias, vmag=4.0):
+        worst = 0.0
+        for gap in torch.arange(8.0, 30.0, 0.25):
+            p_tail = _rtz_fp16(torch.exp2(-gap - bias).reshape(1)).float().item()
+            p_top = _rtz_fp16(torch.exp2(torch.tensor([-bias]))).float().item()
+            got = (p_top * vmag - (L - 1) * p_tail * vmag) / (p_top + (L - 1) * p_tail)
+            w = (L - 1) * 2.0 ** -gap.item()
+            want = (vmag - w * vmag) / (1.0 + w)
+            worst = max(worst, abs(got - want))
+        return worst
+
+    bias = _kernel_bias_log2()
+    assert bias <= 0.0
+    for L in (4096, 16384, 65536):
+        assert worst_error(L, bias) <= 2.5e-3
+    assert worst_error(16384, 6.0) > 0.1          # what the bound protects against
+    assert _rtz_fp16(torch.tensor([1.0 + 2.0 ** -11, 3.9999, 2.0 ** -25])).tolist() == [1.0, 3.998046875, 0.0]
