@@ -12,7 +12,8 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libfused_attn_gfx950.so")
 
 # every symbol include/fused_attn.h declares
-EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_strided", "fa_fwd_plan", "fa_fwd_query", "fa_strerror", "fa_fwd_timed")
+EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_strided", "fa_fwd_plan", "fa_fwd_query", "fa_strerror", "fa_fwd_timed",
+           "fa_qkv_proj")
 FLAG_CAUSAL = 1
 FLAG_BF16 = 2
 
@@ -49,6 +50,8 @@ def load_library():
     lib.fa_fwd_strided.restype = ctypes.c_int
     lib.fa_fwd_timed.argtypes = fwd_args + [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
     lib.fa_fwd_timed.restype = ctypes.c_int
+    lib.fa_qkv_proj.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, vp, ctypes.c_int, vp]
+    lib.fa_qkv_proj.restype = ctypes.c_int
     lib.fa_fwd_plan.argtypes = [i64, i64, i64, i64, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int)]
     lib.fa_fwd_plan.restype = ctypes.c_int
     lib.fa_fwd_query.argtypes = [i64]
@@ -217,3 +220,54 @@ def forward_timed(q, k, v, head_dim, out, iters, mask=None, layout="blf", scale=
             int(iters), ctypes.byref(ms))
     _check(status)
     return float(ms.value)
+
+
+def qkv_project(x, w, num_heads, head_dim, bias=None, rope=None, out=None):
+    """fa_qkv_proj on torch GPU tensors, on torch's current stream: x [B, L, F_in] times w
+    [F_in, 3 * num_heads * head_dim] (+ bias) -> packed [B, L, 3, num_heads * head_dim] (fp16 or
+    bf16, like x).  rope = (cos, sin), float32 [L, head_dim / 2] tables of a rotate-half rotary
+    encoding applied to the q and k slices.  The three slices out[:, :, s] are views that
+    `forward` takes as q, k and v without a copy."""
+    import torch
+
+    for name, t in (("x", x), ("w", w), ("bias", bias), ("out", out)):
+        if t is not None and not isinstance(t, torch.Tensor):
+            raise TypeError("%s must be a torch.Tensor, got %s" % (name, type(t).__name__))
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("x must be float16 or bfloat16, got %s" % x.dtype)
+    if x.dim() != 3 or w.dim() != 2:
+        raise ValueError("x must be [B, L, F_in] and w [F_in, 3 F]")
+    B, L, f_in = x.shape
+    F = num_heads * head_dim
+    if tuple(w.shape) != (f_in, 3 * F):
+        raise ValueError("w must have shape [F_in, 3 * num_heads * head_dim] = [%d, %d], got %s"
+                         % (f_in, 3 * F, tuple(w.shape)))
+    if bias is not None and tuple(bias.shape) != (3 * F,):
+        raise ValueError("bias must have shape [%d], got %s" % (3 * F, tuple(bias.shape)))
+    if out is None:
+        out = torch.empty((B, L, 3, F), dtype=x.dtype, device=x.device)
+    elif tuple(out.shape) != (B, L, 3, F):
+        raise ValueError("out must have shape [%d, %d, 3, %d], got %s" % (B, L, F, tuple(out.shape)))
+    tables = (None, None)
+    if rope is not None:
+        tables = tuple(rope)
+        for name, t in zip(("rope cos", "rope sin"), tables):
+            if not isinstance(t, torch.Tensor) or t.dtype != torch.float32 or tuple(t.shape) != (L, head_dim // 2):
+                raise ValueError("%s must be a float32 tensor of shape [%d, %d]" % (name, L, head_dim // 2))
+    for name, t in (("x", x), ("w", w), ("bias", bias), ("out", out), ("rope cos", tables[0]), ("rope sin", tables[1])):
+        if t is None:
+            continue
+        if name in ("w", "bias", "out") and t.dtype != x.dtype:
+            raise TypeError("%s must have the dtype of x (%s), got %s" % (name, x.dtype, t.dtype))
+        if not t.is_contiguous():
+            raise ValueError("%s must be contiguous" % name)
+        if not t.is_cuda or t.device != x.device:
+            raise ValueError("%s must be on the GPU of x, got device %s" % (name, t.device))
+    flags = FLAG_BF16 if x.dtype == torch.bfloat16 else 0
+    with torch.cuda.device(x.device):
+        status = load_library().fa_qkv_proj(
+            x.data_ptr(), w.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(),
+            B, L, f_in, num_heads, head_dim, tables[0].data_ptr() if rope is not None else None,
+            tables[1].data_ptr() if rope is not None else None, flags, _current_stream(x) or None)
+    _check(status)
+    return out

@@ -3,6 +3,7 @@
 // include/fused_attn.cuh:860-894): picks the workgroup shape, sizes the dynamic LDS block,
 // builds the grid and launches on the caller's stream.
 #include "fused_attn_kernel.hpp"
+#include "qkv_proj_kernel.hpp"
 
 #include "../../include/fused_attn.h"
 
@@ -427,6 +428,75 @@ int fa_fwd_timed(const void* q, const void* k, const void* v, const void* mask, 
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     return rc;
+}
+
+}  // extern "C"
+
+namespace {
+template <int HR, bool BF>
+hipError_t launch_qkv(const fa::qkv::Params& p, hipStream_t stream) {
+    auto kernel = fa::qkv::qkv_proj_kernel<HR, BF>;
+    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), fa::qkv::kLdsBytes);
+    if (e != hipSuccess) return e;
+    fa::qkv::Params params = p;
+    void* args[] = {&params};
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(p.wgs_per_xcd * fa::kNumXcd),
+                           dim3(fa::qkv::kWaves * 64), args, fa::qkv::kLdsBytes, stream);
+}
+
+template <bool BF>
+hipError_t dispatch_qkv(int64_t rope_head_dim, const fa::qkv::Params& p, hipStream_t stream) {
+    switch (rope_head_dim) {
+        case 0: return launch_qkv<0, BF>(p, stream);
+        case 16: return launch_qkv<16, BF>(p, stream);
+        case 32: return launch_qkv<32, BF>(p, stream);
+        case 64: return launch_qkv<64, BF>(p, stream);
+        case 128: return launch_qkv<128, BF>(p, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+}  // namespace
+
+extern "C" {
+
+int fa_qkv_proj(const void* x, const void* w, const void* bias, void* qkv, int64_t B, int64_t L, int64_t F_in,
+                int64_t R, int64_t H, const float* rope_cos, const float* rope_sin, int flags, void* stream) {
+    if ((flags & ~FA_FLAG_BF16) != 0) return FA_ERR_BAD_FLAGS;
+    if (x == nullptr || w == nullptr || qkv == nullptr) return FA_ERR_NULL_POINTER;
+    if ((rope_cos == nullptr) != (rope_sin == nullptr)) return FA_ERR_NULL_POINTER;
+    if (!fa_fwd_query(H)) return FA_ERR_BAD_HEAD_DIM;
+    if (B < 1 || L < 1 || R < 1 || F_in < 1) return FA_ERR_BAD_SHAPE;
+    constexpr int64_t kMaxInt = 0x7fffffff;
+    if (B > kMaxInt || L > kMaxInt || R > kMaxInt || B * L > kMaxInt - 2 * fa::qkv::kTileM) return FA_ERR_TOO_LARGE;
+    const int64_t F = R * H;
+    // the contraction is walked in whole steps of 64, and the three slices start on 64-feature boundaries
+    if (F_in % fa::qkv::kTileK != 0 || F % 64 != 0) return FA_ERR_BAD_SHAPE;
+    // the loaders keep 32-bit byte offsets inside a tile: 256 rows of x, 64 rows of w
+    if (F_in > ((int64_t)1 << 22) || F > ((int64_t)1 << 22)) return FA_ERR_TOO_LARGE;
+    if (!aligned16(x) || !aligned16(w) || !aligned16(qkv) || !aligned16(rope_cos) || !aligned16(rope_sin) ||
+        (reinterpret_cast<uintptr_t>(bias) & 7u) != 0)
+        return FA_ERR_MISALIGNED;
+    fa::qkv::Params p;
+    p.x = static_cast<const _Float16*>(x);
+    p.w = static_cast<const _Float16*>(w);
+    p.bias = static_cast<const _Float16*>(bias);
+    p.out = static_cast<_Float16*>(qkv);
+    p.rope_cos = rope_cos;
+    p.rope_sin = rope_sin;
+    p.M = (int)(B * L);
+    p.K = (int)F_in;
+    p.N = (int)(3 * F);
+    p.F = (int)F;
+    p.L = (int)L;
+    const int64_t tiles_m = ceil_div(B * L, fa::qkv::kTileM);
+    p.tiles_n = (int)ceil_div(3 * F, fa::qkv::kTileN);
+    if (tiles_m * p.tiles_n > kMaxInt - 8) return FA_ERR_TOO_LARGE;
+    p.total_wgs = (int)(tiles_m * p.tiles_n);
+    p.wgs_per_xcd = (int)ceil_div(p.total_wgs, fa::kNumXcd);
+    const int64_t hr = rope_cos != nullptr ? H : 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const hipError_t e = (flags & FA_FLAG_BF16) != 0 ? dispatch_qkv<true>(hr, p, s) : dispatch_qkv<false>(hr, p, s);
+    return static_cast<int>(e);
 }
 
 }  // extern "C"

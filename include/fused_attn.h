@@ -134,6 +134,26 @@ int fa_fwd_timed(const void* q, const void* k, const void* v, const void* mask, 
                  int64_t stride_b, int64_t stride_h, int64_t stride_l,
                  float scale, void* stream, int iters, float* ms_per_launch);
 
+/*
+ * Fused QKV projection, the front end the reference lists as not done (reference README.md:137;
+ * its kernel takes queries, keys and values as three separate tensors, reference
+ * src/fused_attn_extention.cu:15-22):
+ *     qkv[b, l, s, :] = x[b, l, :] w[:, s F : (s + 1) F] (+ bias[s F : (s + 1) F]),   s = 0, 1, 2,  F = R H
+ * x is [B, L, F_in], w is [F_in, 3 F] (input features along the rows), bias (nullable) is [3 F], qkv
+ * is the packed [B, L, 3, F] tensor, all contiguous, fp16 (bfloat16 with FA_FLAG_BF16), f32
+ * accumulation, one rounding.  The three slices qkv[:, :, s, :] are what fa_fwd_strided takes as q,
+ * k and v (stride_b = 3 L F, stride_h = H, stride_l = 3 F) without a copy.
+ * rope_cos / rope_sin (both or neither; nullable): float32 [L, H / 2] tables of a rotary position
+ * encoding in the rotate-half form, applied to every head of the q and k slices before the rounding:
+ *     out[i] = y[i] cos[l, i] - y[i + H/2] sin[l, i],  out[i + H/2] = y[i + H/2] cos[l, i] + y[i] sin[l, i]
+ * for i < H / 2, y the projected head vector.
+ * F_in and F must be multiples of 64 (FA_ERR_BAD_SHAPE otherwise); x, w, qkv and the tables 16-byte
+ * aligned, bias 8-byte aligned.  Launches on `stream` and returns without synchronising.
+ */
+int fa_qkv_proj(const void* x, const void* w, const void* bias, void* qkv,
+                int64_t B, int64_t L, int64_t F_in, int64_t R, int64_t H,
+                const float* rope_cos, const float* rope_sin, int flags, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

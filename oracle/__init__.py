@@ -7,3 +7,4 @@ The product path (fused_attention_amd, module fused_attn) never falls back to it
 """
 from .naive_attention import (attention, attention_f64, attention_lse, attention_per_head,  # noqa: F401
                               causal_mask)
+from .qkv_projection import qkv_projection, rope_tables, rotate_half  # noqa: F401

@@ -12,7 +12,8 @@ import numpy as np
 import pytest
 import torch
 
-from oracle import attention, attention_f64, attention_lse, attention_per_head, causal_mask
+from oracle import (attention, attention_f64, attention_lse, attention_per_head, causal_mask, qkv_projection,
+                    rope_tables, rotate_half)
 
 ORACLE_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle")
 
@@ -244,3 +245,76 @@ def test_rounding_model_of_small_weights():
         assert worst_error(L, bias) <= 2.5e-3
     assert worst_error(16384, 6.0) > 0.1          # what the bound protects against
     assert _rtz_fp16(torch.tensor([1.0 + 2.0 ** -11, 3.9999, 2.0 ** -25])).tolist() == [1.0, 3.998046875, 0.0]
+
+
+# ---- the QKV projection front end and the rotary encoding ----------------------------------------
+
+def test_projection_is_the_library_linear_map_and_its_slices_are_q_k_v():
+    B, L, Fin, R, H = 2, 37, 96, 3, 32
+    F = R * H
+    x, w, b = _rand((B, L, Fin), 900), _rand((Fin, 3 * F), 901, 0.1), _rand((3 * F,), 902)
+    got = qkv_projection(x, w, b, R, H)
+    assert got.shape == (B, L, 3, F) and got.dtype == torch.float32
+    lib = torch.nn.functional.linear(x.float(), w.float().T, b.float()).view(B, L, 3, F)
+    torch.testing.assert_close(got, lib, rtol=1e-5, atol=1e-5)
+    ref64 = (np.einsum("blk,kn->bln", x.double().numpy(), w.double().numpy()) + b.double().numpy()).reshape(B, L, 3, F)
+    assert np.abs(got.numpy() - ref64).max() < 1e-4
+    # slice s of the output uses columns [s F, (s + 1) F) of w
+    for s in range(3):
+        only = qkv_projection(x, w[:, s * F:(s + 1) * F].repeat(1, 3), None, R, H)
+        torch.testing.assert_close(only[:, :, 0], got[:, :, s] - b.float()[s * F:(s + 1) * F], rtol=1e-5, atol=1e-5)
+
+
+def test_projection_closed_forms():
+    B, L, R, H = 1, 9, 2, 32
+    F = R * H
+    x = _rand((B, L, F), 910)
+    eye3 = torch.eye(F).repeat(1, 3).half()
+    out = qkv_projection(x, eye3, None, R, H)                      # identity weights: the input three times
+    for s in range(3):
+        assert torch.equal(out[:, :, s], x.float())
+    w = torch.zeros(F, 3 * F)
+    w[5, 0], w[7, F + 1], w[11, 2 * F + 2] = 1.0, 2.0, -1.0        # one-hot columns pick input features
+    out = qkv_projection(x, w.half(), None, R, H)
+    assert torch.equal(out[0, :, 0, 0], x[0, :, 5].float())
+    assert torch.equal(out[0, :, 1, 1], 2.0 * x[0, :, 7].float())
+    assert torch.equal(out[0, :, 2, 2], -x[0, :, 11].float())
+    assert out.abs().sum() == out[0, :, 0, 0].abs().sum() + out[0, :, 1, 1].abs().sum() + out[0, :, 2, 2].abs().sum()
+
+
+def test_rotary_encoding_is_a_rotation_of_feature_pairs():
+    L, H = 50, 64
+    cos, sin = rope_tables(L, H)
+    assert torch.equal(cos[0], torch.ones(H // 2)) and torch.equal(sin[0], torch.zeros(H // 2))
+    inv = 10000.0 ** (-2.0 * torch.arange(H // 2, dtype=torch.float64) / H)
+    torch.testing.assert_close(cos[7].double(), torch.cos(7 * inv), rtol=0, atol=1e-6)
+    y = _rand((3, L, H), 920).float()
+    out = rotate_half(y, cos, sin)
+    # an independent formulation: (y[i], y[i + H/2]) as a complex number, multiplied by exp(i theta)
+    z = torch.complex(y[..., :H // 2].double(), y[..., H // 2:].double()) * torch.polar(
+        torch.ones(L, H // 2, dtype=torch.float64), torch.atan2(sin.double(), cos.double()))
+    torch.testing.assert_close(out.double(), torch.cat([z.real, z.imag], dim=-1), rtol=0, atol=1e-5)
+    torch.testing.assert_close(out.norm(dim=-1), y.norm(dim=-1), rtol=1e-5, atol=1e-5)        # rotations keep norms
+    assert torch.equal(rotate_half(y, torch.ones_like(cos), torch.zeros_like(sin)), y)
+    # q at position m times k at position n depends on m - n only
+    q, k = _rand((H,), 921).float(), _rand((H,), 922).float()
+
+    def score(m, n):
+        return (rotate_half(q, cos[m], sin[m]) * rotate_half(k, cos[n], sin[n])).sum()
+
+    assert abs(score(9, 4) - score(25, 20)) < 1e-3 and abs(score(9, 4) - score(4, 9)) > 1e-3
+
+
+def test_projection_rotates_q_and_k_heads_only():
+    B, L, Fin, R, H = 2, 21, 64, 3, 16
+    F = R * H
+    x, w, b = _rand((B, L, Fin), 930), _rand((Fin, 3 * F), 931, 0.2), _rand((3 * F,), 932)
+    cos, sin = rope_tables(L, H)
+    plain = qkv_projection(x, w, b, R, H)
+    rot = qkv_projection(x, w, b, R, H, cos, sin)
+    assert torch.equal(rot[:, :, 2], plain[:, :, 2])                                        # v untouched
+    torch.testing.assert_close(rot[:, 0], plain[:, 0], rtol=0, atol=1e-6)                   # position 0: no rotation
+    for s in range(2):
+        for h in range(R):
+            want = rotate_half(plain[:, :, s, h * H:(h + 1) * H], cos.view(1, L, H // 2), sin.view(1, L, H // 2))
+            torch.testing.assert_close(rot[:, :, s, h * H:(h + 1) * H], want, rtol=0, atol=1e-6)
