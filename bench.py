@@ -8,7 +8,13 @@ evaluation of the same workload timed on the host cores over a bounded sample of
 pairs.  Counterpart of the reference's benchmark (reference tests/benchmark_fused_attn.py:8-45),
 which prints wall-clock milliseconds of 128 naive and 128 fused launches.
 
+Before the counted warm-up the step is launched for half a second, so that the chip's clock has
+settled ("settle_launches").  With the default workload the line also carries "workloads": kernel
+time, TFLOP/s, roofline fraction and error on a bounded sample for the other configurations and for
+the QKV projection front end.
+
 usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5a|c5b|readme] [--causal]
+                       [--others auto|on|off]
 """
 import argparse
 import json
@@ -139,6 +145,60 @@ def side_workload(name, dev, check_budget_s):
     return entry
 
 
+def projection_workload(name, dev, rope):
+    """The fused QKV projection front end (fa_qkv_proj) at the feature sizes of a benchmark
+    configuration: hidden [B, L, R*H] times weight [R*H, 3*R*H] into the packed qkv tensor the
+    attention kernel reads.  Kernel time from events on the launch stream (torch's current stream);
+    flop = 2 * B*L * R*H * 3*R*H; error against the float32 oracle on a sample of rows."""
+    import math
+
+    import torch
+
+    from fused_attention_amd import capi, workloads
+    from oracle import qkv_projection, rope_tables
+
+    w = workloads.WORKLOADS[name]
+    F = w.R * w.H
+    gen = torch.Generator().manual_seed(w.seed * 1000 + 7)
+    x = torch.randn(w.B, w.L, F, generator=gen).to(torch.float16)
+    wt = (torch.randn(F, 3 * F, generator=gen) / math.sqrt(F)).to(torch.float16)
+    tables = rope_tables(w.L, w.H) if rope else None
+    xd, wd = x.to(dev), wt.to(dev)
+    td = tuple(t.to(dev) for t in tables) if rope else None
+    out = torch.empty(w.B, w.L, 3, F, dtype=torch.float16, device=dev)
+
+    def step():
+        return capi.qkv_project(xd, wd, w.R, w.H, rope=td, out=out)
+
+    flop = 2.0 * w.B * w.L * F * 3 * F
+    step()
+    torch.cuda.synchronize()
+    iters = max(20, min(2000, int(0.3 / (flop / 0.9e15))))
+    for _ in range(iters):
+        step()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    kernel_ms = e0.elapsed_time(e1) / iters
+    rows = torch.arange(0, w.L, max(1, w.L // 64))
+    want = qkv_projection(x[:1, rows], wt, None, w.R, w.H, *((tables[0][rows], tables[1][rows]) if rope else (None, None)))
+    got = out[:1, rows.to(dev)].float().cpu()
+    tflops = flop / (kernel_ms * 1e-3) / 1e12
+    return {
+        "shape": "B=%d L=%d F_in=%d R=%d H=%d%s" % (w.B, w.L, F, w.R, w.H, " rotary" if rope else ""),
+        "kernel_ms": kernel_ms,
+        "launches_timed": iters,
+        "tflops": tflops,
+        "frac": tflops / PEAK_TFLOPS_FP16,
+        "max_abs_err": (got - want).abs().max().item(),
+        "finite": bool(torch.isfinite(out.float()).all()),
+        "rows_checked": int(rows.numel()),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -263,6 +323,10 @@ def main():
         torch.cuda.empty_cache()
         line["workloads"] = {name: side_workload(name, dev, args.check_budget_s)
                              for name in OTHER_WORKLOADS if name != args.workload}
+        # the projection front end at the headline's and the reference benchmark's feature sizes
+        line["workloads"]["qkv_proj_c3"] = projection_workload("c3", dev, rope=False)
+        line["workloads"]["qkv_proj_c3_rotary"] = projection_workload("c3", dev, rope=True)
+        line["workloads"]["qkv_proj_readme"] = projection_workload("readme", dev, rope=False)
     print(json.dumps(line))
 
 

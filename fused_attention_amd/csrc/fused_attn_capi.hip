@@ -322,7 +322,8 @@ const char* fa_strerror(int status) {
         case FA_OK: return "success";
         case FA_ERR_NULL_POINTER: return "fa_fwd: q, k, v and out must be non-null device pointers";
         case FA_ERR_BAD_HEAD_DIM: return "fa_fwd: head_dim must be 16, 32, 64 or 128";
-        case FA_ERR_BAD_SHAPE: return "fa_fwd: B, R and L must be at least 1";
+        case FA_ERR_BAD_SHAPE:
+            return "fa_fwd: B, R and L must be at least 1 (fa_qkv_proj: and the feature counts multiples of 64)";
         case FA_ERR_BAD_STRIDE:
             return "fa_fwd: strides must be non-negative multiples of 8 elements and stride_l >= head_dim";
         case FA_ERR_MISALIGNED: return "fa_fwd: q, k, v and out must be 16-byte aligned";

@@ -104,10 +104,63 @@ torch::Tensor attention_forward(int64_t head_dim, int64_t chunk_size, torch::Ten
     return output;
 }
 
+// The projection in front of the attention kernel, which the reference lists as not done (reference
+// README.md:137): hidden [batch, seq_len, in_features] times weight [in_features, 3 * num_heads *
+// head_dim] (+ bias) -> packed [batch, seq_len, 3, num_heads * head_dim], optionally with a rotary
+// position encoding (float32 [seq_len, head_dim / 2] cos and sin tables) on the q and k slices.
+torch::Tensor qkv_projection(torch::Tensor hidden, torch::Tensor weight, std::optional<torch::Tensor> bias,
+                             int64_t num_heads, int64_t head_dim, std::optional<torch::Tensor> rope_cos,
+                             std::optional<torch::Tensor> rope_sin) {
+    TORCH_CHECK(hidden.dtype() == torch::kFloat16 || hidden.dtype() == torch::kBFloat16,
+                "hidden must be float16 or bfloat16, got ", hidden.dtype());
+    TORCH_CHECK(hidden.device().type() == torch::kCUDA, "hidden must be a GPU tensor, got device ", hidden.device());
+    TORCH_CHECK(hidden.dim() == 3 && hidden.is_contiguous(), "hidden must be a contiguous 3-D tensor");
+    TORCH_CHECK(fa_fwd_query(head_dim) == 1 && num_heads >= 1, "head_dim must be 16, 32, 64 or 128 and num_heads >= 1");
+    const int64_t batch_size = hidden.size(0), seq_len = hidden.size(1), in_features = hidden.size(2);
+    const int64_t num_features = num_heads * head_dim;
+    auto same_kind = [&](const torch::Tensor& t, const char* name) {
+        TORCH_CHECK(t.dtype() == hidden.dtype() && t.device() == hidden.device() && t.is_contiguous(), name,
+                    " must be a contiguous tensor with the dtype and device of hidden");
+    };
+    same_kind(weight, "weight");
+    TORCH_CHECK(weight.dim() == 2 && weight.size(0) == in_features && weight.size(1) == 3 * num_features,
+                "weight must have shape [in_features, 3 * num_heads * head_dim] = [", in_features, ", ",
+                3 * num_features, "], got ", weight.sizes());
+    const void* bias_ptr = nullptr;
+    if (bias.has_value()) {
+        same_kind(*bias, "bias");
+        TORCH_CHECK(bias->dim() == 1 && bias->size(0) == 3 * num_features, "bias must have shape [", 3 * num_features, "]");
+        bias_ptr = bias->data_ptr();
+    }
+    TORCH_CHECK(rope_cos.has_value() == rope_sin.has_value(), "rope_cos and rope_sin go together");
+    const float* cos_ptr = nullptr;
+    const float* sin_ptr = nullptr;
+    if (rope_cos.has_value()) {
+        for (const torch::Tensor* t : {&*rope_cos, &*rope_sin})
+            TORCH_CHECK(t->dtype() == torch::kFloat32 && t->device() == hidden.device() && t->is_contiguous() &&
+                            t->dim() == 2 && t->size(0) == seq_len && t->size(1) == head_dim / 2,
+                        "rope tables must be contiguous float32 [seq_len, head_dim / 2] tensors on the device of hidden");
+        cos_ptr = rope_cos->data_ptr<float>();
+        sin_ptr = rope_sin->data_ptr<float>();
+    }
+    const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(hidden.device());
+    torch::Tensor qkv = torch::empty({batch_size, seq_len, 3, num_features}, hidden.options());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(hidden.device().index()).stream();
+    const int status = fa_qkv_proj(hidden.data_ptr(), weight.data_ptr(), bias_ptr, qkv.data_ptr(), batch_size, seq_len,
+                                   in_features, num_heads, head_dim, cos_ptr, sin_ptr,
+                                   hidden.dtype() == torch::kBFloat16 ? FA_FLAG_BF16 : 0, static_cast<void*>(stream));
+    TORCH_CHECK(status == FA_OK, "fused QKV projection failed: ", fa_strerror(status));
+    return qkv;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("attention_forward", &attention_forward, py::arg("head_dim"), py::arg("chunk_size"),
           py::arg("queries"), py::arg("keys"), py::arg("values"),
           py::arg("mask") = std::optional<torch::Tensor>(), "Fused multihead attention");
+    m.def("qkv_projection", &qkv_projection, py::arg("hidden"), py::arg("weight"),
+          py::arg("bias") = std::optional<torch::Tensor>(), py::arg("num_heads"), py::arg("head_dim"),
+          py::arg("rope_cos") = std::optional<torch::Tensor>(), py::arg("rope_sin") = std::optional<torch::Tensor>(),
+          "Fused QKV projection into the packed [batch, seq_len, 3, num_heads * head_dim] tensor");
 }

@@ -8,9 +8,10 @@
 // (reference src/fused_attn_extention.cu:15-22).
 //
 // One kernel, one pass: a workgroup of eight wave64s owns a 256 x 256 tile of the output and walks
-// the contraction in steps of 64.  x and w tiles stream through a two-stage LDS ring written by
-// direct-to-LDS loads (16 bytes per lane, no staging registers), laid out column-major in 16-byte
-// chunks like the K/V rings of the attention kernel (kColStride).  The products are computed
+// the contraction in steps of 64.  x and w tiles go global -> registers -> LDS with 16-byte
+// accesses, whole cache lines per wave on the global side, into two LDS stages of row-major tiles
+// with padded rows (the loads of the next step are in flight while this one is consumed).  The
+// products are computed
 // transposed, C^T = W^T X^T, with v_mfma_f32_32x32x16_f16: the A operand W^T (32 outputs n x 16 k)
 // comes from the row-major w tile through the LDS transpose read (ds_read_b64_tr_b16), the B
 // operand X^T (16 k x 32 rows m) is a plain 16-byte read of a row of x.  In the accumulator a lane
@@ -31,10 +32,15 @@ constexpr int kTileM = 256;
 constexpr int kTileN = 256;
 constexpr int kTileK = 64;
 constexpr int kWaves = 8;
-// one 64-row x 16-byte block of a ring tile, in halves (1 KB plus the pad of the attention rings)
-constexpr int kBlk = kColStride;
-constexpr int kXTile = (kTileK / 8) * (kTileM / 64) * kBlk;   // chunk c, row block rb at (c * 4 + rb) * kBlk
-constexpr int kWTile = (kTileN / 8) * kBlk;                   // feature chunk cn at cn * kBlk, 64 k rows each
+constexpr int kBand = 4;      // row tiles per band of the tile order
+// LDS tiles are row-major with padded rows, so that the 16-byte operand reads of x (32 consecutive
+// rows per half-wave) and the transpose reads of w (four contraction rows x 32 bytes per 16 lanes)
+// touch every bank once: 144-byte rows of x put 16 consecutive rows on distinct 16-byte bank
+// groups, 576-byte rows of w put four consecutive rows 16 banks apart.
+constexpr int kXStr = kTileK + 8;                   // halves per row of the x tile [256][64]
+constexpr int kWStr = kTileN + 32;                  // halves per row of the w tile [64][256]
+constexpr int kXTile = kTileM * kXStr;
+constexpr int kWTile = kTileK * kWStr;
 constexpr int kLdsBytes = 2 * (kXTile + kWTile) * (int)sizeof(_Float16);
 
 struct Params {
@@ -68,45 +74,61 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
     const int wm = wave >> 1;          // which 64 rows of the tile
     const int wn = wave & 1;           // which 128 features of the tile
 
-    // Workgroups are dealt round-robin to the XCDs: renumber so that one XCD receives consecutive
-    // tiles, which share their rows of x (the feature tiles of one row tile follow each other).
+    // Workgroups are dealt round-robin to the XCDs: renumber so that one XCD (one L2) receives
+    // consecutive tiles, and order the tiles in bands of four row tiles, feature tile by feature
+    // tile inside a band: the 32 workgroups resident on an XCD then cover about 4 x 8 tiles and
+    // share 4 row blocks of x and 8 column blocks of w in L2, instead of 1 and 32.
     const int wg = blockIdx.x;
     const int logical = (wg % kNumXcd) * p.wgs_per_xcd + wg / kNumXcd;
     if (logical >= p.total_wgs) return;
-    const int m0 = (logical / p.tiles_n) * kTileM;
-    const int n0 = (logical % p.tiles_n) * kTileN;
+    const int tiles_m = p.total_wgs / p.tiles_n;
+    const int band = logical / (kBand * p.tiles_n);
+    const int in_band = logical - band * (kBand * p.tiles_n);
+    const int band_rows = min(kBand, tiles_m - band * kBand);
+    const int m0 = (band * kBand + in_band % band_rows) * kTileM;
+    const int n0 = (in_band / band_rows) * kTileN;
 
-    // ---- loads: every wave fetches four x blocks and four w blocks of a stage -------------------
-    // x block (c, rb): lane l = row m0 + rb 64 + l, 16 bytes at k chunk c.  Rows beyond M are read
-    // from row M - 1 (their results are never stored).  w block cn: lane l = contraction row
-    // k0 + l, 16 bytes at feature chunk cn; chunks beyond N are not fetched (their LDS block then
-    // holds stale data that only reaches output features which are never stored).
-    uint32_t xoff[4], woff[4];
-    uint32_t xlds[4], wlds[4];
-    bool wvalid[4];
+    // ---- loads: global -> registers -> LDS, 16 bytes per lane ------------------------------------
+    // x tile: chunk idx = tid + 512 i is row idx / 8, 16-byte chunk idx % 8: eight lanes read the 128
+    // bytes of one row, a wave reads eight whole cache lines per instruction.  Rows beyond M are
+    // read from row M - 1 (their results are never stored).  w tile: chunk idx is contraction row
+    // idx / 32, feature chunk idx % 32: 32 lanes read 512 contiguous bytes of a row; chunks beyond N
+    // are not fetched and hold zeros.
+    constexpr int NP = 4;      // chunks per thread and tile, of x and of w
+    uint32_t xoff[NP], woff[NP], xdst[NP], wdst[NP];
+    bool wvalid[NP];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int blk = wave * 4 + i;               // 0..31
-        const int c = blk >> 2, rb = blk & 3;
-        const int row = min(m0 + rb * 64 + lane, p.M - 1) - m0;
-        xoff[i] = ((uint32_t)row * (uint32_t)p.K + (uint32_t)c * 8u) * 2u;
-        xlds[i] = (uint32_t)(c * 4 + rb) * (kBlk * 2);
-        const int cn = blk;
-        woff[i] = ((uint32_t)lane * (uint32_t)p.N + (uint32_t)cn * 8u) * 2u;
-        wlds[i] = (uint32_t)cn * (kBlk * 2);
-        wvalid[i] = n0 + cn * 8 < p.N;
+    for (int i = 0; i < NP; ++i) {
+        const int idx = tid + i * (kWaves * 64);
+        const int row = min(m0 + (idx >> 3), p.M - 1) - m0;
+        xoff[i] = ((uint32_t)row * (uint32_t)p.K + (uint32_t)(idx & 7) * 8u) * 2u;
+        xdst[i] = (uint32_t)((idx >> 3) * kXStr + (idx & 7) * 8);
+        woff[i] = ((uint32_t)(idx >> 5) * (uint32_t)p.N + (uint32_t)(idx & 31) * 8u) * 2u;
+        wdst[i] = (uint32_t)((idx >> 5) * kWStr + (idx & 31) * 8);
+        wvalid[i] = n0 + (idx & 31) * 8 < p.N;
     }
-    const _Float16* xsrc = p.x + (int64_t)m0 * p.K;                 // k0 = 0
-    const _Float16* wsrc = p.w + n0;
-    const uint32_t xs_addr = (uint32_t)(uintptr_t)(FA_LDS void*)xs;
-    const uint32_t ws_addr = (uint32_t)(uintptr_t)(FA_LDS void*)ws;
-    auto issue = [&](int stage) __attribute__((always_inline)) {
+    const char* xsrc = reinterpret_cast<const char*>(p.x + (int64_t)m0 * p.K);     // advanced by every fetch
+    const char* wsrc = reinterpret_cast<const char*>(p.w + n0);
+    // two sets of staging registers: a tile is fetched two steps before it is consumed
+    u32x4 xreg[2][NP], wreg[2][NP];
+    auto fetch = [&](auto set_c) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_c)::value;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            RingLoader<64, 4>::dma16(xs_addr + stage * (kXTile * 2) + xlds[i], xsrc, xoff[i]);
+        for (int i = 0; i < NP; ++i) xreg[SET][i] = *reinterpret_cast<const u32x4*>(xsrc + xoff[i]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (wvalid[i]) RingLoader<64, 4>::dma16(ws_addr + stage * (kWTile * 2) + wlds[i], wsrc, woff[i]);
+        for (int i = 0; i < NP; ++i) {
+            wreg[SET][i] = u32x4{0u, 0u, 0u, 0u};
+            if (wvalid[i]) wreg[SET][i] = *reinterpret_cast<const u32x4*>(wsrc + woff[i]);
+        }
+        xsrc += kTileK * 2;
+        wsrc += (int64_t)kTileK * p.N * 2;
+    };
+    auto stash = [&](auto set_c, int stage) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_c)::value;
+#pragma unroll
+        for (int i = 0; i < NP; ++i) *reinterpret_cast<u32x4*>(xs + stage * kXTile + xdst[i]) = xreg[SET][i];
+#pragma unroll
+        for (int i = 0; i < NP; ++i) *reinterpret_cast<u32x4*>(ws + stage * kWTile + wdst[i]) = wreg[SET][i];
     };
 
     floatx16 acc[4][2];
@@ -118,45 +140,41 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
             for (int r = 0; r < 16; ++r) acc[nt][mt][r] = 0.f;
 
     // per-lane parts of the operand addresses
-    // B operand (x): row wm 64 + mt 32 + ln of chunk 2 s + g
-    const int xrow = wm * 64 + ln;
-    const _Float16* const xop_base = xs + (g * 4 + (xrow >> 6)) * kBlk + (xrow & 63) * 8;
+    // B operand (x): row wm 64 + mt 32 + ln, contraction chunk 2 s + g
+    const _Float16* const xop_base = xs + (wm * 64 + ln) * kXStr + 8 * g;
     // A operand (w^T), transpose read: lane s16 of a 16-lane group points at contraction row
-    // 8 g + s16 / 4 (+ 4 for the second read), halves 4 (s16 % 4) ... of the 32-byte span of features
-    // that starts at chunk 2 * ((lane / 16) % 2); feature block nt adds 4 chunks.  Lane j of the
-    // group receives four consecutive contraction rows of feature j: slot (g, i) of the operand is
-    // contraction index 16 s + 8 g + i, the order in which the 16-byte read of x delivers them.
+    // 8 g + s16 / 4 (+ 4 for the second read), features 4 (s16 % 4) ... of the 16 that start at
+    // 16 * ((lane / 16) % 2); feature block nt adds 32.  Lane j of the group receives four
+    // consecutive contraction rows of feature j: slot (g, i) of the operand is contraction index
+    // 16 s + 8 g + i, the order in which the 16-byte read of x delivers them.
     const int s16 = lane & 15;
-    const _Float16* const wop_base = ws + (wn * 16 + 2 * ((lane >> 4) & 1) + ((s16 & 3) >> 1)) * kBlk +
-                                     (8 * g + (s16 >> 2)) * 8 + 4 * (s16 & 1);
+    const _Float16* const wop_base = ws + (8 * g + (s16 >> 2)) * kWStr + wn * 128 + 16 * ((lane >> 4) & 1) +
+                                     4 * (s16 & 3);
 
+    // Two LDS stages, two register sets.  Step kt consumes tile kt from LDS stage kt % 2; the loads of
+    // tile kt + 2 are sent off at its start into register set kt % 2, and at its end tile kt + 1
+    // (requested one step earlier) moves from the other set to the other stage, which everybody
+    // finished reading before the barrier that ended step kt - 1.
     const int ksteps = p.K / kTileK;
-    issue(0);
-    wait_ring_loads();
-    __syncthreads();
-    for (int kt = 0; kt < ksteps; ++kt) {
-        const int stage = kt & 1;
-        if (kt + 1 < ksteps) {
-            xsrc += kTileK;
-            wsrc += (int64_t)kTileK * p.N;
-            issue(stage ^ 1);
-        }
-        const _Float16* const xb = xop_base + stage * kXTile;
-        const _Float16* const wb = wop_base + stage * kWTile;
+    auto step = [&](int kt, auto par_c) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(par_c)::value;
+        if (kt + 2 < ksteps) fetch(std::integral_constant<int, PAR>{});
+        const _Float16* const xb = xop_base + PAR * kXTile;
+        const _Float16* const wb = wop_base + PAR * kWTile;
 #pragma unroll
         for (int s = 0; s < kTileK / 16; ++s) {
             half8 wop[4], xop[2];
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt) {
-                const _Float16* p0 = wb + nt * 4 * kBlk + (16 * s) * 8;
+                const _Float16* p0 = wb + (16 * s) * kWStr + nt * 32;
                 const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS short4v*)(p0));
-                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS short4v*)(p0 + 4 * 8));
+                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS short4v*)(p0 + 4 * kWStr));
                 const short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 wop[nt] = __builtin_bit_cast(half8, both);
             }
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
-                xop[mt] = *reinterpret_cast<const half8*>(xb + (2 * s) * 4 * kBlk + mt * 32 * 8);
+                xop[mt] = *reinterpret_cast<const half8*>(xb + mt * 32 * kXStr + s * 16);
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
@@ -167,10 +185,16 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
                         acc[nt][mt] = mfma32(wop[nt], xop[mt], acc[nt][mt]);
                 }
         }
-        // this wave's loads of the next stage have landed; after the barrier everybody's have, and
-        // everybody is done reading the stage that the loads after next will overwrite
-        wait_ring_loads();
+        if (kt + 1 < ksteps) stash(std::integral_constant<int, 1 - PAR>{}, 1 - PAR);
         __syncthreads();
+    };
+    fetch(std::integral_constant<int, 0>{});
+    stash(std::integral_constant<int, 0>{}, 0);
+    if (ksteps > 1) fetch(std::integral_constant<int, 1>{});
+    __syncthreads();
+    for (int kt = 0; kt < ksteps; kt += 2) {
+        step(kt, std::integral_constant<int, 0>{});
+        if (kt + 1 < ksteps) step(kt + 1, std::integral_constant<int, 1>{});
     }
 
     // ---- epilogue: bias, rotation, one rounding, 8-byte stores ------------------------------------

@@ -133,3 +133,20 @@ def test_projection_rejections(gpu):
         capi.qkv_project(x, w, 1, 64, rope=(torch.zeros(64, 16, device=gpu), torch.zeros(64, 32, device=gpu)))
     with pytest.raises(ValueError, match="GPU of x"):
         capi.qkv_project(x, w.cpu(), 1, 64)
+
+
+def test_projection_through_the_torch_binding(gpu):
+    import fused_attn
+
+    B, L, Fin, R, H = 2, 200, 128, 2, 64
+    x, w, b = _rand((B, L, Fin), 7500), _rand((Fin, 3 * R * H), 7501, 0.1), _rand((3 * R * H,), 7502)
+    cos, sin = rope_tables(L, H)
+    got = fused_attn.qkv_projection(x.to(gpu), w.to(gpu), b.to(gpu), R, H, cos.to(gpu), sin.to(gpu))
+    assert got.shape == (B, L, 3, R * H) and got.dtype == torch.float16 and got.device.type == "cuda"
+    _close(got, qkv_projection(x, w, b, R, H, cos, sin))
+    same = capi.qkv_project(x.to(gpu), w.to(gpu), R, H, bias=b.to(gpu), rope=(cos.to(gpu), sin.to(gpu)))
+    assert torch.equal(got, same)
+    with pytest.raises(RuntimeError, match="weight must have shape"):
+        fused_attn.qkv_projection(x.to(gpu), w[:, :64].contiguous().to(gpu), None, R, H)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        fused_attn.qkv_projection(x, w, None, R, H)
