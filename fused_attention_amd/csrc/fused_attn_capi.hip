@@ -492,7 +492,9 @@ int fa_qkv_proj(const void* x, const void* w, const void* bias, void* qkv, int64
     const int64_t tiles_m = ceil_div(B * L, fa::qkv::kTileM);
     p.tiles_n = (int)ceil_div(3 * F, fa::qkv::kTileN);
     if (tiles_m * p.tiles_n > kMaxInt - 8) return FA_ERR_TOO_LARGE;
-    p.total_wgs = (int)(tiles_m * p.tiles_n);
+    p.total_tiles = (int)(tiles_m * p.tiles_n);
+    // a resident grid, one workgroup per compute unit, each walking through its share of the tiles
+    p.total_wgs = p.total_tiles < kNumCu ? p.total_tiles : kNumCu;
     p.wgs_per_xcd = (int)ceil_div(p.total_wgs, fa::kNumXcd);
     const int64_t hr = rope_cos != nullptr ? H : 0;
     hipStream_t s = static_cast<hipStream_t>(stream);

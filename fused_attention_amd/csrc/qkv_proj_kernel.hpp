@@ -54,8 +54,9 @@ struct Params {
     int F;                   // features per slice (N = 3 F)
     int L;                   // sequence length: position of row m is m % L
     int tiles_n;             // ceil(N / 256)
-    int total_wgs;           // tiles_m * tiles_n
-    int wgs_per_xcd;
+    int total_tiles;         // tiles_m * tiles_n
+    int total_wgs;           // workgroups that take tiles: min(total_tiles, one per compute unit)
+    int wgs_per_xcd;         // ceil(total_wgs / 8): the grid is 8 times this
 };
 
 // HR = head_dim of the rotation (16, 32, 64, 128), or 0 for none.
@@ -74,19 +75,22 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
     const int wm = wave >> 1;          // which 64 rows of the tile
     const int wn = wave & 1;           // which 128 features of the tile
 
-    // Workgroups are dealt round-robin to the XCDs: renumber so that one XCD (one L2) receives
-    // consecutive tiles, and order the tiles in bands of four row tiles, feature tile by feature
-    // tile inside a band: the 32 workgroups resident on an XCD then cover about 4 x 8 tiles and
-    // share 4 row blocks of x and 8 column blocks of w in L2, instead of 1 and 32.
+    // A resident grid: workgroup `logical` takes the tiles logical, logical + G, logical + 2 G, ...
+    // Workgroups are dealt round-robin to the XCDs, so they are renumbered first: one XCD (one L2)
+    // then works on consecutive tiles, and the tiles are ordered in bands of four row tiles, feature
+    // tile by feature tile inside a band: the 32 workgroups of an XCD cover about 4 x 8 tiles at a
+    // time and share 4 row blocks of x and 8 column blocks of w in L2, instead of 1 and 32.
     const int wg = blockIdx.x;
     const int logical = (wg % kNumXcd) * p.wgs_per_xcd + wg / kNumXcd;
     if (logical >= p.total_wgs) return;
-    const int tiles_m = p.total_wgs / p.tiles_n;
-    const int band = logical / (kBand * p.tiles_n);
-    const int in_band = logical - band * (kBand * p.tiles_n);
-    const int band_rows = min(kBand, tiles_m - band * kBand);
-    const int m0 = (band * kBand + in_band % band_rows) * kTileM;
-    const int n0 = (in_band / band_rows) * kTileN;
+    const int tiles_m = p.total_tiles / p.tiles_n;
+    auto tile_origin = [&](int tile, int& m0, int& n0) __attribute__((always_inline)) {
+        const int band = tile / (kBand * p.tiles_n);
+        const int in_band = tile - band * (kBand * p.tiles_n);
+        const int band_rows = min(kBand, tiles_m - band * kBand);
+        m0 = (band * kBand + in_band % band_rows) * kTileM;
+        n0 = (in_band / band_rows) * kTileN;
+    };
 
     // ---- loads: global -> registers -> LDS, 16 bytes per lane ------------------------------------
     // x tile: chunk idx = tid + 512 i is row idx / 8, 16-byte chunk idx % 8: eight lanes read the 128
@@ -94,22 +98,37 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
     // read from row M - 1 (their results are never stored).  w tile: chunk idx is contraction row
     // idx / 32, feature chunk idx % 32: 32 lanes read 512 contiguous bytes of a row; chunks beyond N
     // are not fetched and hold zeros.
+    // The loads run ahead of the arithmetic as one stream over all (tile, contraction step) pairs of
+    // the workgroup: the first steps of the next tile are on their way while this one is finished.
     constexpr int NP = 4;      // chunks per thread and tile, of x and of w
     uint32_t xoff[NP], woff[NP], xdst[NP], wdst[NP];
     bool wvalid[NP];
+    const char* xsrc = nullptr;
+    const char* wsrc = nullptr;
+    int fetch_tile = logical, fetch_kt = 0;
+    auto aim = [&]() __attribute__((always_inline)) {      // point the loads at the first step of fetch_tile
+        int m0, n0;
+        tile_origin(fetch_tile, m0, n0);
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            const int idx = tid + i * (kWaves * 64);
+            const int row = min(m0 + (idx >> 3), p.M - 1) - m0;
+            xoff[i] = ((uint32_t)row * (uint32_t)p.K + (uint32_t)(idx & 7) * 8u) * 2u;
+            wvalid[i] = n0 + (idx & 31) * 8 < p.N;
+        }
+        xsrc = reinterpret_cast<const char*>(p.x + (int64_t)m0 * p.K);
+        wsrc = reinterpret_cast<const char*>(p.w + n0);
+    };
 #pragma unroll
     for (int i = 0; i < NP; ++i) {
         const int idx = tid + i * (kWaves * 64);
-        const int row = min(m0 + (idx >> 3), p.M - 1) - m0;
-        xoff[i] = ((uint32_t)row * (uint32_t)p.K + (uint32_t)(idx & 7) * 8u) * 2u;
         xdst[i] = (uint32_t)((idx >> 3) * kXStr + (idx & 7) * 8);
         woff[i] = ((uint32_t)(idx >> 5) * (uint32_t)p.N + (uint32_t)(idx & 31) * 8u) * 2u;
         wdst[i] = (uint32_t)((idx >> 5) * kWStr + (idx & 31) * 8);
-        wvalid[i] = n0 + (idx & 31) * 8 < p.N;
     }
-    const char* xsrc = reinterpret_cast<const char*>(p.x + (int64_t)m0 * p.K);     // advanced by every fetch
-    const char* wsrc = reinterpret_cast<const char*>(p.w + n0);
-    // two sets of staging registers: a tile is fetched two steps before it is consumed
+    aim();
+    const int ksteps = p.K / kTileK;
+    // two sets of staging registers: a step's data is fetched two steps before it is consumed
     u32x4 xreg[2][NP], wreg[2][NP];
     auto fetch = [&](auto set_c) __attribute__((always_inline)) {
         constexpr int SET = decltype(set_c)::value;
@@ -122,6 +141,11 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
         }
         xsrc += kTileK * 2;
         wsrc += (int64_t)kTileK * p.N * 2;
+        if (++fetch_kt == ksteps) {
+            fetch_kt = 0;
+            fetch_tile += p.total_wgs;
+            if (fetch_tile < p.total_tiles) aim();
+        }
     };
     auto stash = [&](auto set_c, int stage) __attribute__((always_inline)) {
         constexpr int SET = decltype(set_c)::value;
@@ -151,14 +175,103 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
     const _Float16* const wop_base = ws + (8 * g + (s16 >> 2)) * kWStr + wn * 128 + 16 * ((lane >> 4) & 1) +
                                      4 * (s16 & 3);
 
-    // Two LDS stages, two register sets.  Step kt consumes tile kt from LDS stage kt % 2; the loads of
-    // tile kt + 2 are sent off at its start into register set kt % 2, and at its end tile kt + 1
-    // (requested one step earlier) moves from the other set to the other stage, which everybody
-    // finished reading before the barrier that ended step kt - 1.
-    const int ksteps = p.K / kTileK;
-    auto step = [&](int kt, auto par_c) __attribute__((always_inline)) {
+    // ---- end of a tile: bias, rotation, one rounding, 8-byte stores; the accumulators start over ---
+    // acc[nt][mt][r]: row m = m0 + wm 64 + mt 32 + ln, feature n = n0 + wn 128 + nt 32 + 8 (r / 4) + 4 g + r % 4.
+    // The accumulators are only read here (results are formed in temporaries): modifying them in
+    // place inside the step loop makes the compiler carry a second copy of all of them.
+    auto finish_tile = [&](int done_tile) __attribute__((always_inline)) {
+        int m0, n0;
+        tile_origin(done_tile, m0, n0);
+        const int nw = n0 + wn * 128;
+        // one run of four features of one row: bias added, rounded, stored
+        auto biased = [&](int nt, int mt, int r4, int n) __attribute__((always_inline)) {
+            floatx4 v = {acc[nt][mt][4 * r4], acc[nt][mt][4 * r4 + 1], acc[nt][mt][4 * r4 + 2], acc[nt][mt][4 * r4 + 3]};
+            if (p.bias != nullptr && n < p.N) {
+                const u16x4 b4 = *reinterpret_cast<const u16x4*>(p.bias + n);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += BF ? bf16::elem_to_float(b4[e]) : elem_to_float(b4[e]);
+            }
+            return v;
+        };
+        auto store_run = [&](floatx4 v, int m, int n) __attribute__((always_inline)) {
+            if (m < p.M && n < p.N) {
+                u16x4 hv;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) hv[e] = BF ? bf16::float_to_elem(v[e]) : float_to_elem(v[e]);
+                *reinterpret_cast<u32x2*>(p.out + (int64_t)m * p.N + n) = __builtin_bit_cast(u32x2, hv);
+            }
+        };
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+            const int m = m0 + wm * 64 + mt * 32 + ln;
+            if constexpr (HR > 0) {
+                // rotate-half: within a head, feature i < HR / 2 pairs with feature i + HR / 2:
+                //   out[i] = y[i] cos_i - y[i + HR/2] sin_i,  out[i + HR/2] = y[i + HR/2] cos_i + y[i] sin_i
+                // with cos_i, sin_i taken at the row's position m % L.  Only the q and k slices (n < 2 F).
+                const int pos = (m < p.M ? m : p.M - 1) % p.L;
+                const float* const cs = p.rope_cos + (int64_t)pos * (HR / 2);
+                const float* const sn = p.rope_sin + (int64_t)pos * (HR / 2);
+#pragma unroll
+                for (int pr = 0; pr < 8; ++pr) {       // the 16 runs a lane holds per row form 8 pairs
+                    int nt_a, r4_a, nt_b, r4_b;
+                    if constexpr (HR == 128) {          // head = the wave's 128 features: block nt pairs with nt + 2
+                        nt_a = pr >> 2; r4_a = pr & 3; nt_b = nt_a + 2; r4_b = r4_a;
+                    } else if constexpr (HR == 64) {    // head = two blocks: nt pairs with nt + 1
+                        nt_a = 2 * (pr >> 2); r4_a = pr & 3; nt_b = nt_a + 1; r4_b = r4_a;
+                    } else if constexpr (HR == 32) {    // head = one block: register group r4 pairs with r4 + 2
+                        nt_a = pr >> 1; r4_a = pr & 1; nt_b = nt_a; r4_b = r4_a + 2;
+                    } else {                            // head = half a block: register group r4 pairs with r4 + 1
+                        nt_a = pr >> 1; r4_a = 2 * (pr & 1); nt_b = nt_a; r4_b = r4_a + 1;
+                    }
+                    const int n_a = nw + nt_a * 32 + 8 * r4_a + 4 * g;      // first features of the two runs
+                    const int n_b = nw + nt_b * 32 + 8 * r4_b + 4 * g;
+                    floatx4 a = biased(nt_a, mt, r4_a, n_a);
+                    floatx4 b = biased(nt_b, mt, r4_b, n_b);
+                    if (n_a < 2 * p.F) {
+                        const int i0 = n_a % (HR / 2);      // index inside the half head
+                        const floatx4 c4 = *reinterpret_cast<const floatx4*>(cs + i0);
+                        const floatx4 s4 = *reinterpret_cast<const floatx4*>(sn + i0);
+                        const floatx4 ra = a * c4 - b * s4;
+                        const floatx4 rb = b * c4 + a * s4;
+                        a = ra;
+                        b = rb;
+                    }
+                    store_run(a, m, n_a);
+                    store_run(b, m, n_b);
+                    // one pair at a time: all table loads at once would not fit in the registers
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; ++r4) {
+                        const int n = nw + nt * 32 + 8 * r4 + 4 * g;
+                        store_run(biased(nt, mt, r4, n), m, n);
+                    }
+            }
+        }
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[nt][mt][r] = 0.f;
+    };
+
+    // Two LDS stages, two register sets.  Step t of the workgroup's stream consumes its data from LDS
+    // stage t % 2; the loads of step t + 2 are sent off at its start into register set t % 2, and at
+    // its end the data of step t + 1 (requested one step earlier) moves from the other set to the
+    // other stage, which everybody finished reading before the barrier that ended step t - 1.
+    const int my_tiles = (p.total_tiles - logical + p.total_wgs - 1) / p.total_wgs;
+    const int total_steps = my_tiles * ksteps;
+    int tile = logical, kt = 0;
+    auto step = [&](int t, auto par_c) __attribute__((always_inline)) {
         constexpr int PAR = decltype(par_c)::value;
-        if (kt + 2 < ksteps) fetch(std::integral_constant<int, PAR>{});
+        // (at the last step of a tile the loads are sent off behind the epilogue instead, so that no
+        // staging register is live while the epilogue needs registers of its own)
+        const bool last = kt + 1 == ksteps;
+        if (!last && t + 2 < total_steps) fetch(std::integral_constant<int, PAR>{});
         const _Float16* const xb = xop_base + PAR * kXTile;
         const _Float16* const wb = wop_base + PAR * kWTile;
 #pragma unroll
@@ -185,90 +298,24 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
                         acc[nt][mt] = mfma32(wop[nt], xop[mt], acc[nt][mt]);
                 }
         }
-        if (kt + 1 < ksteps) stash(std::integral_constant<int, 1 - PAR>{}, 1 - PAR);
+        if (t + 1 < total_steps) stash(std::integral_constant<int, 1 - PAR>{}, 1 - PAR);
         __syncthreads();
+        if (last) {
+            finish_tile(tile);
+            kt = 0;
+            tile += p.total_wgs;
+            if (t + 2 < total_steps) fetch(std::integral_constant<int, PAR>{});
+        } else {
+            ++kt;
+        }
     };
     fetch(std::integral_constant<int, 0>{});
     stash(std::integral_constant<int, 0>{}, 0);
-    if (ksteps > 1) fetch(std::integral_constant<int, 1>{});
+    if (total_steps > 1) fetch(std::integral_constant<int, 1>{});
     __syncthreads();
-    for (int kt = 0; kt < ksteps; kt += 2) {
-        step(kt, std::integral_constant<int, 0>{});
-        if (kt + 1 < ksteps) step(kt + 1, std::integral_constant<int, 1>{});
-    }
-
-    // ---- epilogue: bias, rotation, one rounding, 8-byte stores ------------------------------------
-    // acc[nt][mt][r]: row m = m0 + wm 64 + mt 32 + ln, feature n = n0 + wn 128 + nt 32 + 8 (r / 4) + 4 g + r % 4
-    const int nw = n0 + wn * 128;
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
-        const int m = m0 + wm * 64 + mt * 32 + ln;
-        if (p.bias != nullptr) {
-#pragma unroll
-            for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    const int n = nw + nt * 32 + 8 * r4 + 4 * g;
-                    if (n < p.N) {
-                        const u16x4 b4 = *reinterpret_cast<const u16x4*>(p.bias + n);
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            acc[nt][mt][4 * r4 + e] += BF ? bf16::elem_to_float(b4[e]) : elem_to_float(b4[e]);
-                    }
-                }
-        }
-        if constexpr (HR > 0) {
-            // rotate-half: within a head, feature i < HR / 2 pairs with feature i + HR / 2:
-            //   out[i] = x[i] cos_i - x[i + HR/2] sin_i,  out[i + HR/2] = x[i + HR/2] cos_i + x[i] sin_i
-            // with cos_i, sin_i taken at the row's position m % L.  Only the q and k slices (n < 2 F).
-            const int pos = (m < p.M ? m : p.M - 1) % p.L;
-            const float* const cs = p.rope_cos + (int64_t)pos * (HR / 2);
-            const float* const sn = p.rope_sin + (int64_t)pos * (HR / 2);
-            // (block, register group) of the first half and of its partner, by head_dim
-            constexpr int NPAIR = 8;   // the 16 runs of four features a lane holds per row form 8 pairs
-#pragma unroll
-            for (int pr = 0; pr < NPAIR; ++pr) {
-                int nt_a, r4_a, nt_b, r4_b;
-                if constexpr (HR == 128) {          // head = the wave's 128 features: block nt pairs with nt + 2
-                    nt_a = pr >> 2; r4_a = pr & 3; nt_b = nt_a + 2; r4_b = r4_a;
-                } else if constexpr (HR == 64) {    // head = two blocks: nt pairs with nt + 1
-                    nt_a = 2 * (pr >> 2); r4_a = pr & 3; nt_b = nt_a + 1; r4_b = r4_a;
-                } else if constexpr (HR == 32) {    // head = one block: register group r4 pairs with r4 + 2
-                    nt_a = pr >> 1; r4_a = pr & 1; nt_b = nt_a; r4_b = r4_a + 2;
-                } else {                            // head = half a block: register group r4 pairs with r4 + 1
-                    nt_a = pr >> 1; r4_a = 2 * (pr & 1); nt_b = nt_a; r4_b = r4_a + 1;
-                }
-                const int n_a = nw + nt_a * 32 + 8 * r4_a + 4 * g;      // first feature of the run in the first half
-                if (n_a < 2 * p.F) {
-                    const int i0 = n_a % (HR / 2);      // index inside the half head
-                    const floatx4 c4 = *reinterpret_cast<const floatx4*>(cs + i0);
-                    const floatx4 s4 = *reinterpret_cast<const floatx4*>(sn + i0);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float a = acc[nt_a][mt][4 * r4_a + e];
-                        const float b = acc[nt_b][mt][4 * r4_b + e];
-                        acc[nt_a][mt][4 * r4_a + e] = a * c4[e] - b * s4[e];
-                        acc[nt_b][mt][4 * r4_b + e] = b * c4[e] + a * s4[e];
-                    }
-                }
-            }
-        }
-        if (m < p.M) {
-            _Float16* const orow = p.out + (int64_t)m * p.N;
-#pragma unroll
-            for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    const int n = nw + nt * 32 + 8 * r4 + 4 * g;
-                    if (n < p.N) {
-                        u16x4 hv;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            hv[e] = BF ? bf16::float_to_elem(acc[nt][mt][4 * r4 + e]) : float_to_elem(acc[nt][mt][4 * r4 + e]);
-                        *reinterpret_cast<u32x2*>(orow + n) = __builtin_bit_cast(u32x2, hv);
-                    }
-                }
-        }
+    for (int t = 0; t < total_steps; t += 2) {
+        step(t, std::integral_constant<int, 0>{});
+        if (t + 1 < total_steps) step(t + 1, std::integral_constant<int, 1>{});
     }
 }
 
