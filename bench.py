@@ -35,7 +35,9 @@ PEAK_TFLOPS_FP16 = 2500.0   # MI355X dense fp16 MFMA, published
 # counter run report null.
 MEASURED_TRAFFIC = {
     "c3": (134.4e6, "profiles/fwd_kernel_pingpong_c3.md"),
-    "c4": (808.2e6, "profiles/fwd_kernel_pingpong_c4.md"),
+    "c4": (806.7e6, "profiles/fwd_kernel_pingpong_c4.md"),
+    "qkv_proj_c3": (271.8e6, "profiles/qkv_proj_kernel_c3.md"),
+    "qkv_proj_readme": (2187.5e6, "profiles/qkv_proj_kernel_readme.md"),
 }
 
 # Launches made before the counted warm-up until this much time has passed: the chip needs a few
@@ -145,7 +147,7 @@ def side_workload(name, dev, check_budget_s):
     return entry
 
 
-def projection_workload(name, dev, rope):
+def projection_workload(name, dev, rope, iters=None):
     """The fused QKV projection front end (fa_qkv_proj) at the feature sizes of a benchmark
     configuration: hidden [B, L, R*H] times weight [R*H, 3*R*H] into the packed qkv tensor the
     attention kernel reads.  Kernel time from events on the launch stream (torch's current stream);
@@ -173,7 +175,8 @@ def projection_workload(name, dev, rope):
     flop = 2.0 * w.B * w.L * F * 3 * F
     step()
     torch.cuda.synchronize()
-    iters = max(20, min(2000, int(0.3 / (flop / 0.9e15))))
+    if iters is None:
+        iters = max(20, min(2000, int(0.3 / (flop / 0.9e15))))
     for _ in range(iters):
         step()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -196,6 +199,9 @@ def projection_workload(name, dev, rope):
         "max_abs_err": (got - want).abs().max().item(),
         "finite": bool(torch.isfinite(out.float()).all()),
         "rows_checked": int(rows.numel()),
+        "bytes_algorithmic": (w.B * w.L * F + F * 3 * F + w.B * w.L * 3 * F) * 2,
+        "traffic": None if rope else MEASURED_TRAFFIC.get("qkv_proj_" + name, (None, None))[0],
+        "traffic_source": None if rope else MEASURED_TRAFFIC.get("qkv_proj_" + name, (None, None))[1],
     }
 
 
@@ -212,6 +218,9 @@ def main():
                     help="size of the plain copy run before the timed region (0 disables it)")
     ap.add_argument("--cpu-budget-s", type=float, default=15.0,
                     help="seconds of host time for the CPU baseline sample (0 disables it)")
+    ap.add_argument("--projection", choices=["plain", "rotary"], default=None,
+                    help="measure the fused QKV projection front end at the workload's feature sizes "
+                         "instead of the attention forward (one JSON line, flop = 2*B*L*F*3F)")
     ap.add_argument("--others", choices=["auto", "on", "off"], default="auto",
                     help="also measure the other benchmark configurations into \"workloads\" "
                          "(auto: with the default headline workload, non-causal)")
@@ -232,10 +241,6 @@ def main():
     capi.load_library()     # fail loudly if the kernel library is not built
     w = workloads.WORKLOADS[args.workload]
     dev = torch.device("cuda:0")
-    q, k, v = workloads.make_inputs(w)
-    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
-    chunk = min(128, w.H * 2)
-
     # A plain device-to-device copy of known size, outside the timed region: the reference point
     # against which the HBM counters (FETCH_SIZE / WRITE_SIZE) of a profiler run are scaled.
     if args.calibration_copy_mib > 0:
@@ -245,6 +250,21 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if args.projection:
+        entry = projection_workload(args.workload, dev, rope=args.projection == "rotary", iters=args.steps)
+        print(json.dumps({
+            "metric": "fused qkv projection TFLOP/s (2*B*L*F*3F)", "value": entry["tflops"], "unit": "TFLOP/s",
+            "n_gpus": 1, "steps": entry["launches_timed"], "warmup": entry["launches_timed"],
+            "ms_per_step": entry["kernel_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f16", "data": "synthetic", "config": {"workload": "qkv projection, " + entry["shape"]},
+            "roofline": {"bound": "mfma", "achieved": entry["tflops"], "peak": PEAK_TFLOPS_FP16, "unit": "TFLOP/s",
+                         "frac": entry["frac"], "traffic": None, "kernel_ms": entry["kernel_ms"]},
+            "max_abs_err": entry["max_abs_err"]}))
+        return
+    q, k, v = workloads.make_inputs(w)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    chunk = min(128, w.H * 2)
 
     if args.causal:
         out = torch.empty_like(qd)
