@@ -56,6 +56,12 @@ extern "C" {
  * 1/sqrt(head_dim) (reference include/fused_attn.cuh:727).
  * B, R, L >= 1.  L*stride_l, R*stride_h and B*stride_b must stay below 2^62 elements and
  * stride_l must not exceed 2^24 elements (FA_ERR_TOO_LARGE otherwise).
+ * Accuracy: scores, softmax state and both products are accumulated in float32; the softmax
+ * weights are rounded to fp16 before they multiply the values, scaled so that a key at the row
+ * maximum weighs 16.  A key more than 28 log2 units (19.4 natural-log units) below the largest
+ * score of its row therefore contributes nothing, and a row of L keys loses at most L * 2^-28 of
+ * its weight (2.4e-4 at L = 65536).  The reference accumulates everything in fp16 (reference
+ * include/fused_attn.cuh:174,257,650-653).
  */
 int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* out,
            int64_t B, int64_t R, int64_t L, int64_t H,
