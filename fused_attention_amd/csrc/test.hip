@@ -6,6 +6,7 @@
 // softmax(Q K^T / sqrt(H)) V and exits non-zero when the error exceeds the tolerance.
 //
 // usage: fa_test [B R L H [iters [blhd|bhld [input_scale [qzero|vconst|vcol]]]]]
+//        fa_test qkv [B L R H [iters]]   the projection front end (fa_qkv_proj, bias + rotary encoding)
 //        fa_test mfma-peak        what v_mfma_f32_32x32x16_f16 sustains on this chip with zero
 //                                 operands and with N(0,1) operands (the rate depends on the data)
 #include <hip/hip_runtime.h>
@@ -138,6 +139,100 @@ void fill_values(std::vector<_Float16>& dst, uint32_t seed, float amp) {
     }
 }
 
+// fa_test qkv B L R H [iters]: the projection front end (fa_qkv_proj) with generator-filled x, w and
+// bias and a rotary encoding, sampled rows checked against a double-precision host evaluation.
+int qkv_check(int64_t B, int64_t L, int64_t R, int64_t H, int iters) {
+    const int64_t F = R * H, M = B * L, N = 3 * F;
+    std::printf("fa_test qkv B=%lld L=%lld F_in=%lld R=%lld H=%lld\n", (long long)B, (long long)L, (long long)F,
+                (long long)R, (long long)H);
+    std::vector<_Float16> x(M * F), w(F * N), bias(N), out(M * N);
+    fill_values(x, 179u, 1.7320508f);
+    fill_values(w, 1791u, 1.7320508f / std::sqrt((float)F));
+    fill_values(bias, 17917u, 1.0f);
+    std::vector<float> cs(L * (H / 2)), sn(L * (H / 2));
+    for (int64_t l = 0; l < L; ++l)
+        for (int64_t i = 0; i < H / 2; ++i) {
+            const double angle = (double)l * std::pow(10000.0, -2.0 * (double)i / (double)H);
+            cs[l * (H / 2) + i] = (float)std::cos(angle);
+            sn[l * (H / 2) + i] = (float)std::sin(angle);
+        }
+    _Float16 *dx, *dw, *db, *dout;
+    float *dcs, *dsn;
+    HIP_OK(hipMalloc(&dx, x.size() * 2));
+    HIP_OK(hipMalloc(&dw, w.size() * 2));
+    HIP_OK(hipMalloc(&db, bias.size() * 2));
+    HIP_OK(hipMalloc(&dout, out.size() * 2));
+    HIP_OK(hipMalloc(&dcs, cs.size() * 4));
+    HIP_OK(hipMalloc(&dsn, sn.size() * 4));
+    HIP_OK(hipMemcpy(dx, x.data(), x.size() * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dw, w.data(), w.size() * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(db, bias.data(), bias.size() * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dcs, cs.data(), cs.size() * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dsn, sn.data(), sn.size() * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemset(dout, 0xff, out.size() * 2));
+    int rc = fa_qkv_proj(dx, dw, db, dout, B, L, F, R, H, dcs, dsn, 0, nullptr);
+    if (rc != 0) {
+        std::fprintf(stderr, "fa_qkv_proj: %s\n", fa_strerror(rc));
+        return 2;
+    }
+    HIP_OK(hipDeviceSynchronize());
+    HIP_OK(hipMemcpy(out.data(), dout, out.size() * 2, hipMemcpyDeviceToHost));
+    int64_t nonfinite = 0, checked = 0;
+    for (const _Float16 v : out)
+        if (!std::isfinite((float)v)) ++nonfinite;
+    double max_ratio = 0.0, max_err = 0.0;      // error over its tolerance 2e-3 + 1e-3 |want|, and the error itself
+    std::vector<double> y(N);
+    const int64_t step = M > 48 ? M / 41 + 1 : 1;
+    for (int64_t m = 0; m < M; m += (m + step < M || m == M - 1) ? step : M - 1 - m) {
+        for (int64_t n = 0; n < N; ++n) {
+            double acc = (double)(float)bias[n];
+            for (int64_t k = 0; k < F; ++k) acc += (double)(float)x[m * F + k] * (double)(float)w[k * N + n];
+            y[n] = acc;
+        }
+        const int64_t l = m % L;
+        for (int64_t n = 0; n < N; ++n) {
+            double want = y[n];
+            if (n < 2 * F) {                                   // q and k slices: rotate-half within the head
+                const int64_t hn = n % H, i = hn % (H / 2);
+                const double c = cs[l * (H / 2) + i], s_ = sn[l * (H / 2) + i];
+                want = hn < H / 2 ? y[n] * c - y[n + H / 2] * s_ : y[n] * c + y[n - H / 2] * s_;
+            }
+            const double err = std::fabs(want - (double)(float)out[m * N + n]);
+            const double ratio = err / (2e-3 + 1e-3 * std::fabs(want));
+            if (!(err <= max_err)) max_err = err;
+            if (!(ratio <= max_ratio)) max_ratio = ratio;
+        }
+        ++checked;
+    }
+    std::printf("checked %lld rows: max abs err %.3e, at most %.2f of the tolerance 2e-3 + 1e-3 |want|, non-finite outputs %lld\n",
+                (long long)checked, max_err, max_ratio, (long long)nonfinite);
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    for (int i = 0; i < 3 && rc == 0; ++i) rc = fa_qkv_proj(dx, dw, db, dout, B, L, F, R, H, dcs, dsn, 0, nullptr);
+    HIP_OK(hipEventRecord(e0, nullptr));
+    for (int i = 0; i < iters && rc == 0; ++i) rc = fa_qkv_proj(dx, dw, db, dout, B, L, F, R, H, dcs, dsn, 0, nullptr);
+    HIP_OK(hipEventRecord(e1, nullptr));
+    HIP_OK(hipEventSynchronize(e1));
+    if (rc != 0) {
+        std::fprintf(stderr, "fa_qkv_proj: %s\n", fa_strerror(rc));
+        return 2;
+    }
+    float ms = 0.f;
+    HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+    ms /= (float)iters;
+    std::printf("%.4f ms per launch, %.1f TFLOP/s (2*B*L*F*3F / t)\n", ms, 2.0 * M * F * N / (ms * 1e-3) / 1e12);
+    (void)hipFree(dx);
+    (void)hipFree(dw);
+    (void)hipFree(db);
+    (void)hipFree(dout);
+    (void)hipFree(dcs);
+    (void)hipFree(dsn);
+    const bool ok = max_ratio <= 1.0 && nonfinite == 0;
+    std::printf("%s\n", ok ? "PASS" : "FAIL");
+    return ok ? 0 : 1;
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -146,6 +241,10 @@ int main(int argc, char** argv) {
     bool bhld = false;
     float amp = 1.7320508f;  // uniform with unit variance
     if (argc >= 2 && std::strcmp(argv[1], "mfma-peak") == 0) return mfma_peak();
+    if (argc >= 2 && std::strcmp(argv[1], "qkv") == 0)
+        return qkv_check(argc >= 3 ? std::atoll(argv[2]) : 2, argc >= 4 ? std::atoll(argv[3]) : 300,
+                         argc >= 5 ? std::atoll(argv[4]) : 4, argc >= 6 ? std::atoll(argv[5]) : 64,
+                         argc >= 7 ? std::atoi(argv[6]) : 20);
     if (argc >= 5) {
         B = std::atoll(argv[1]);
         R = std::atoll(argv[2]);

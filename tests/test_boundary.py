@@ -176,6 +176,34 @@ def test_binding_signature_matches_the_reference():
     assert "Fused multihead attention" in doc
 
 
+def test_binding_exposes_the_projection_front_end():
+    import fused_attn
+
+    doc = fused_attn.qkv_projection.__doc__
+    names = re.findall(r"(\w+): ", doc.split("->")[0])
+    assert names == ["hidden", "weight", "bias", "num_heads", "head_dim", "rope_cos", "rope_sin"]
+    x = torch.zeros(1, 64, 64, dtype=torch.float16)
+    w = torch.zeros(64, 192, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="GPU tensor"):          # host tensors never reach the library
+        fused_attn.qkv_projection(x, w, None, 1, 64)
+    with pytest.raises(RuntimeError, match="float16 or bfloat16"):
+        fused_attn.qkv_projection(x.float(), w.float(), None, 1, 64)
+    with pytest.raises(ValueError, match="GPU of x"):
+        capi.qkv_project(x, w, 1, 64)
+    with pytest.raises(ValueError, match="w must have shape"):
+        capi.qkv_project(x, w[:, :128], 1, 64)
+    lib = capi.load_library()
+    ok = 0x1000   # never dereferenced: rejected during validation
+    assert lib.fa_qkv_proj(ok, ok, None, ok, 1, 64, 96, 1, 64, None, None, 0, None) == -3     # F_in not a multiple of 64
+    assert lib.fa_qkv_proj(ok, ok, None, ok, 1, 64, 64, 3, 16, None, None, 0, None) == -3     # R * H not a multiple of 64
+    assert lib.fa_qkv_proj(ok, ok, None, ok, 1, 64, 64, 1, 48, None, None, 0, None) == -2
+    assert lib.fa_qkv_proj(ok, None, None, ok, 1, 64, 64, 1, 64, None, None, 0, None) == -1
+    assert lib.fa_qkv_proj(ok, ok, None, ok, 1, 64, 64, 1, 64, ok, None, 0, None) == -1        # one table without the other
+    assert lib.fa_qkv_proj(ok, ok + 8, None, ok, 1, 64, 64, 1, 64, None, None, 0, None) == -5
+    assert lib.fa_qkv_proj(ok, ok, None, ok, 1, 64, 64, 1, 64, None, None, 1, None) == -7      # causal is not a projection flag
+    assert lib.fa_qkv_proj(ok, ok, None, ok, 2 ** 20, 2 ** 12, 64, 1, 64, None, None, 0, None) == -6
+
+
 def test_binding_rejects_what_the_reference_rejects():
     import fused_attn
 

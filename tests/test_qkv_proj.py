@@ -150,3 +150,35 @@ def test_projection_through_the_torch_binding(gpu):
         fused_attn.qkv_projection(x.to(gpu), w[:, :64].contiguous().to(gpu), None, R, H)
     with pytest.raises(RuntimeError, match="GPU tensor"):
         fused_attn.qkv_projection(x, w, None, R, H)
+
+
+def test_projection_and_attention_captured_in_one_graph(gpu):
+    # Neither launch allocates or clears anything, so hidden state -> qkv -> attention is recorded as
+    # two kernel nodes; replays follow the contents of the captured input buffer and agree bitwise
+    # with eager launches, with eager work between the replays.
+    B, L, R, H = 2, 512, 8, 64
+    F = R * H
+    x = _rand((B, L, F), 7600).to(gpu)
+    w = _rand((F, 3 * F), 7601, 1.0 / math.sqrt(F)).to(gpu)
+    rope = tuple(t.to(gpu) for t in rope_tables(L, H))
+    qkv = torch.empty(B, L, 3, F, dtype=torch.float16, device=gpu)
+    out = torch.empty(B, L, F, dtype=torch.float16, device=gpu)
+
+    def run(qkv_buf, out_buf):
+        capi.qkv_project(x, w, R, H, rope=rope, out=qkv_buf)
+        capi.forward(qkv_buf[:, :, 0], qkv_buf[:, :, 1], qkv_buf[:, :, 2], H, out=out_buf, causal=True)
+
+    run(qkv, out)                                    # warm-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(qkv, out)
+    for rep in range(3):
+        if rep:
+            x.copy_(_rand((B, L, F), 7610 + rep))
+        qkv_e, out_e = torch.empty_like(qkv), torch.empty_like(out)
+        run(qkv_e, out_e)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(qkv, qkv_e) and torch.equal(out, out_e)
+    _close(qkv, qkv_projection(x.cpu(), w.cpu(), None, R, H, *(t.cpu() for t in rope)))
