@@ -308,6 +308,11 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     p->total_wgs = (int)total;
     p->wgs_per_xcd = (int)((total + fa::kNumXcd - 1) / fa::kNumXcd);
     p->scale_log2e = scale * 1.4426950408889634f;
+    // 11 - ceil(log2 L): a tail of L small weights then loses at most 2^-13 of a row (see kBiasMin)
+    int log2_len = 0;
+    while (((int64_t)1 << log2_len) < L) ++log2_len;
+    const float bias = 11.0f - (float)log2_len;
+    p->bias = bias < fa::kBiasMin ? fa::kBiasMin : (bias > fa::kBiasMax ? fa::kBiasMax : bias);
     return FA_OK;
 }
 

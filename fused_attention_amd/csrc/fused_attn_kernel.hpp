@@ -69,6 +69,7 @@ struct FwdParams {
                            // (t, n - 1 - t) of one head; > 0 = resident grid, the heads of an XCD's
                            // workgroups (B * R / 8 of them) dealt out tile by tile, see the kernel
     float scale_log2e;     // scale * log2(e)
+    float bias;            // bias of the reference of the exponentials, log2 units (see kBiasMin)
 };
 
 constexpr int kNumXcd = 8;
@@ -200,16 +201,19 @@ struct TileLoader {
 // Largest partial row sum (16 terms) the fast path of the online softmax accepts.
 constexpr float kTrip = 16384.f;
 
-// Bias (log2 units) of the reference the exponentials are taken against, in every kernel, and the
-// largest sum of a query's 32 probabilities of one sub-tile that the eight-wave kernel's fast path
-// accepts.  The bias
-// is negative: a key at the reference maximum gets the probability 2^-kBias = 16, so that the
-// fp16 rounding of the probabilities (normal numbers down to 2^-14, subnormals down to 2^-24)
-// reaches 28 log2 units below the maximum before a weight is lost: a tail of L small weights
-// then loses at most L 2^-28 of the row (2.4e-4 at L = 65536).  The reference may lag the true
-// maximum by 15 + kBias = 11 log2 units (10 in the four-wave kernels, whose check works on half
-// rows) before the check sends the wave down the slow path.
-constexpr float kBias = -4.0f;
+// Bias (log2 units) of the reference the exponentials are taken against, in every kernel
+// (FwdParams::bias), and the largest sum of a query's 32 probabilities of one sub-tile that the
+// eight-wave kernel's fast path accepts.  A key at the reference maximum gets the probability
+// 2^-bias.  The probabilities are rounded to fp16 before the second product (normal numbers down
+// to 2^-14, subnormals down to 2^-24), so a weight more than 24 - bias log2 units below the row
+// maximum is lost: a tail of L small weights loses at most L 2^-(24 - bias) of the row.  The
+// launcher picks bias = 11 - ceil(log2 L), between kBiasMin and kBiasMax, which keeps that share
+// at or below 2^-13 = 1.2e-4 whatever the sequence length; what is left of the fp16 range is the
+// leash of the speculative reference, which may lag the true maximum by 15 + bias log2 units (14
+// in the four-wave kernels, whose check works on half rows) before the check sends the wave down
+// the slow path: 14 units at L = 4096, 12 at 16384, 10 at 65536.
+constexpr float kBiasMin = -8.0f;
+constexpr float kBiasMax = 6.0f;
 constexpr float kTripSum = 32768.f;
 
 // O^T[.][nb] *= alpha, in place.  Written as one instruction per register with the register tied

@@ -57,11 +57,11 @@ extern "C" {
  * B, R, L >= 1.  L*stride_l, R*stride_h and B*stride_b must stay below 2^62 elements and
  * stride_l must not exceed 2^24 elements (FA_ERR_TOO_LARGE otherwise).
  * Accuracy: scores, softmax state and both products are accumulated in float32; the softmax
- * weights are rounded to fp16 before they multiply the values, scaled so that a key at the row
- * maximum weighs 16.  A key more than 28 log2 units (19.4 natural-log units) below the largest
- * score of its row therefore contributes nothing, and a row of L keys loses at most L * 2^-28 of
- * its weight (2.4e-4 at L = 65536).  The reference accumulates everything in fp16 (reference
- * include/fused_attn.cuh:174,257,650-653).
+ * weights are rounded to fp16 before they multiply the values, scaled by a power of two chosen
+ * from L so that a row of L keys loses at most 2^-13 (1.2e-4) of its weight to the bottom of the
+ * fp16 range: a key more than 13 + ceil(log2 L) log2 units below the largest score of its row
+ * contributes nothing (25 units, 17 natural-log units, at L = 4096).  The reference accumulates
+ * everything in fp16 (reference include/fused_attn.cuh:174,257,650-653).
  */
 int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* out,
            int64_t B, int64_t R, int64_t L, int64_t H,

@@ -211,23 +211,29 @@ def _rtz_fp16(x):
     return bits.view(torch.float16)
 
 
-def _kernel_bias_log2():
+def _kernel_bias_log2(L):
+    """The launcher's choice (fused_attn_capi.hip): 11 - ceil(log2 L), clamped to the limits the
+    kernel header states."""
     import os
     import re
 
     here = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     text = open(os.path.join(here, "fused_attention_amd", "csrc", "fused_attn_kernel.hpp")).read()
-    return float(re.search(r"constexpr float kBias = (-?[0-9.]+)f;", text).group(1))
+    lo = float(re.search(r"constexpr float kBiasMin = (-?[0-9.]+)f;", text).group(1))
+    hi = float(re.search(r"constexpr float kBiasMax = (-?[0-9.]+)f;", text).group(1))
+    launcher = open(os.path.join(here, "fused_attention_amd", "csrc", "fused_attn_capi.hip")).read()
+    assert "const float bias = 11.0f - (float)log2_len;" in launcher
+    return min(hi, max(lo, 11.0 - math.ceil(math.log2(L))))
 
 
 def test_rounding_model_of_small_weights():
-    # The eight-wave kernel rounds p = exp2(score - reference - bias) toward zero to fp16 before
-    # the second product.  fp16 has normal numbers down to 2^-14 and subnormals down to 2^-24, so
-    # keys more than 24 - bias log2 units below the reference vanish and keys in the ten units
-    # above that are truncated.  Worst case over the gap: one dominant key and L - 1 keys `gap`
-    # below it; the lost share of the row is at most (L - 1) 2^-(24 - bias).  With the bias the
-    # kernel header states, that stays inside half the 5e-3 bound up to L = 65536 for values of
-    # magnitude 4; a bias of +6 (reference 64 times above the maximum) would not.
+    # The kernels round p = exp2(score - reference - bias) toward zero to fp16 before the second
+    # product.  fp16 has normal numbers down to 2^-14 and subnormals down to 2^-24, so keys more
+    # than 24 - bias log2 units below the reference vanish and keys in the ten units above that
+    # are truncated.  Worst case over the gap: one dominant key and L - 1 keys `gap` below it; the
+    # lost share of the row is at most (L - 1) 2^-(24 - bias).  With the bias the launcher picks
+    # for a sequence length, that stays inside half the 5e-3 bound for values of magnitude 4 at
+    # every length; a fixed bias of +6 (reference 64 times above the maximum) would not.
     def worst_error(L, bias, vmag=4.0):
         worst = 0.0
         for gap in torch.arange(8.0, 30.0, 0.25):
@@ -239,10 +245,9 @@ def test_rounding_model_of_small_weights():
             worst = max(worst, abs(got - want))
         return worst
 
-    bias = _kernel_bias_log2()
-    assert bias <= 0.0
-    for L in (4096, 16384, 65536):
-        assert worst_error(L, bias) <= 2.5e-3
+    assert [_kernel_bias_log2(L) for L in (1, 64, 1000, 3073, 4096, 16384, 65536, 2 ** 22)] == [6, 5, 1, -1, -1, -3, -5, -8]
+    for L in (64, 1000, 4096, 16384, 65536, 2 ** 19):
+        assert worst_error(L, _kernel_bias_log2(L)) <= 2.5e-3
     assert worst_error(16384, 6.0) > 0.1          # what the bound protects against
     assert _rtz_fp16(torch.tensor([1.0 + 2.0 ** -11, 3.9999, 2.0 ** -25])).tolist() == [1.0, 3.998046875, 0.0]
 
