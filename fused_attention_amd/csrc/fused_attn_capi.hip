@@ -442,12 +442,14 @@ namespace {
 template <int HR, bool BF>
 hipError_t launch_qkv(const fa::qkv::Params& p, hipStream_t stream) {
     auto kernel = fa::qkv::qkv_proj_kernel<HR, BF>;
-    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), fa::qkv::kLdsBytes);
+    constexpr int kQkvLds = fa::qkv::kLdsBytes;
+    constexpr int kQkvThreads = fa::qkv::kWaves * 64;
+    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), kQkvLds);
     if (e != hipSuccess) return e;
     fa::qkv::Params params = p;
     void* args[] = {&params};
     return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(p.wgs_per_xcd * fa::kNumXcd),
-                           dim3(fa::qkv::kWaves * 64), args, fa::qkv::kLdsBytes, stream);
+                           dim3(kQkvThreads), args, kQkvLds, stream);
 }
 
 template <bool BF>

@@ -8,16 +8,22 @@
 // (reference src/fused_attn_extention.cu:15-22).
 //
 // One kernel, one pass: a workgroup of eight wave64s owns a 256 x 256 tile of the output and walks
-// the contraction in steps of 64.  x and w tiles go global -> registers -> LDS with 16-byte
-// accesses, whole cache lines per wave on the global side, into two LDS stages of row-major tiles
-// with padded rows (the loads of the next step are in flight while this one is consumed).  The
-// products are computed
-// transposed, C^T = W^T X^T, with v_mfma_f32_32x32x16_f16: the A operand W^T (32 outputs n x 16 k)
-// comes from the row-major w tile through the LDS transpose read (ds_read_b64_tr_b16), the B
-// operand X^T (16 k x 32 rows m) is a plain 16-byte read of a row of x.  In the accumulator a lane
-// then owns one output row m and, per 32 x 32 block, 16 output features n in runs of four: bias
-// and rotation are applied in registers (the partner feature n + H/2 of a rotation sits in the
-// same lane), and a run is stored with one 8-byte store.
+// the contraction in slices of 64.  The x and w slices are written into LDS by the loads themselves
+// (direct-to-LDS loads: no staging registers, no LDS store instructions), into a ring of two
+// 64 KB slots.  One load instruction of a wave fills 1 KB of consecutive LDS, lane l the 16 bytes
+// at 16 l, and each lane is free to fetch any 16-byte chunk: the tiles stay row-major without
+// padding, whole cache lines per wave on the global side, and the chunks of a row are permuted
+// (XOR with a few bits of the row index) so that the operand reads touch every bank once:
+//   x slot [256 rows][8 chunks]:  chunk c of row r sits at position c ^ ((r >> 1) & 7)
+//          (16 consecutive rows of one logical chunk cover the 16 bank groups of 16 bytes);
+//   w slot [64 rows][32 chunks]:  chunk c of contraction row k sits at c ^ ((k & 3) << 2)
+//          (the four rows a transpose read touches land in the four 64-byte quarters of the banks).
+// The products are computed transposed, C^T = W^T X^T, with v_mfma_f32_32x32x16_f16: the A operand
+// W^T (32 outputs n x 16 k) comes from the row-major w slice through the LDS transpose read
+// (ds_read_b64_tr_b16), the B operand X^T (16 k x 32 rows m) is a plain 16-byte read of a row of x.
+// In the accumulator a lane then owns one output row m and, per 32 x 32 block, 16 output features
+// n in runs of four: bias and rotation are applied in registers (the partner feature n + H/2 of a
+// rotation sits in the same lane), and a run is stored with one 8-byte store.
 //
 // A wave owns 64 rows x 128 features (4 x 2 blocks of 32 x 32, 128 accumulator registers); its
 // 128 features are whole heads for every head_dim up to 128.
@@ -30,18 +36,11 @@ namespace qkv {
 
 constexpr int kTileM = 256;
 constexpr int kTileN = 256;
-constexpr int kTileK = 64;
+constexpr int kTileK = 64;    // contraction steps per slice (one ring slot)
 constexpr int kWaves = 8;
 constexpr int kBand = 4;      // row tiles per band of the tile order
-// LDS tiles are row-major with padded rows, so that the 16-byte operand reads of x (32 consecutive
-// rows per half-wave) and the transpose reads of w (four contraction rows x 32 bytes per 16 lanes)
-// touch every bank once: 144-byte rows of x put 16 consecutive rows on distinct 16-byte bank
-// groups, 576-byte rows of w put four consecutive rows 16 banks apart.
-constexpr int kXStr = kTileK + 8;                   // halves per row of the x tile [256][64]
-constexpr int kWStr = kTileN + 32;                  // halves per row of the w tile [64][256]
-constexpr int kXTile = kTileM * kXStr;
-constexpr int kWTile = kTileK * kWStr;
-constexpr int kLdsBytes = 2 * (kXTile + kWTile) * (int)sizeof(_Float16);
+constexpr int kSlots = 2;     // ring slots: one is read while the other is filled
+constexpr int kLdsBytes = kSlots * (kTileM + kTileN) * kTileK * (int)sizeof(_Float16);   // 128 KB
 
 struct Params {
     const _Float16* x;       // [M, K]
@@ -59,12 +58,29 @@ struct Params {
     int wgs_per_xcd;         // ceil(total_wgs / 8): the grid is 8 times this
 };
 
+__device__ __forceinline__ void dma16(uint32_t lds_addr, const void* base, uint32_t voff) {
+    // M0 holds the LDS address of lane 0's 16 bytes.  Written in assembly so that the compiler
+    // does not see an LDS write (it would wait for the load before the wave's next LDS read).
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
+
 // HR = head_dim of the rotation (16, 32, 64, 128), or 0 for none.
 template <int HR, bool BF>
 __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p) {
+    constexpr int KS = kTileK;
+    constexpr int NSLOT = kSlots;
+    constexpr int CPRX = KS / 8;                        // 16-byte chunks per row of an x slot
+    constexpr int LX = CPRX / 2;                        // x loads per wave and step
+    constexpr int LW = KS / 16;                         // w loads per wave and step
+    constexpr int XSLOT = kTileM * KS;                  // halves
+    constexpr int WSLOT = KS * kTileN;
+    constexpr int NSUB = KS / 16;                       // 16-wide contraction sub-steps per step
     extern __shared__ __attribute__((aligned(16))) _Float16 smem[];
-    _Float16* const xs = smem;                   // two x tiles
-    _Float16* const ws = smem + 2 * kXTile;      // two w tiles
+    _Float16* const xs = smem;
+    _Float16* const ws = smem + NSLOT * XSLOT;
     typedef short short8v __attribute__((ext_vector_type(8)));
 
     const int tid = threadIdx.x;
@@ -72,8 +88,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 5;
     const int ln = lane & 31;
-    const int wm = wave >> 1;          // which 64 rows of the tile
-    const int wn = wave & 1;           // which 128 features of the tile
+    const int wm = wave >> 1;
+    const int wn = wave & 1;
 
     // A resident grid: workgroup `logical` takes the tiles logical, logical + G, logical + 2 G, ...
     // Workgroups are dealt round-robin to the XCDs, so they are renumbered first: one XCD (one L2)
@@ -92,67 +108,72 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
         n0 = (in_band / band_rows) * kTileN;
     };
 
-    // ---- loads: global -> registers -> LDS, 16 bytes per lane ------------------------------------
-    // x tile: chunk idx = tid + 512 i is row idx / 8, 16-byte chunk idx % 8: eight lanes read the 128
-    // bytes of one row, a wave reads eight whole cache lines per instruction.  Rows beyond M are
-    // read from row M - 1 (their results are never stored).  w tile: chunk idx is contraction row
-    // idx / 32, feature chunk idx % 32: 32 lanes read 512 contiguous bytes of a row; chunks beyond N
-    // are not fetched and hold zeros.
-    // The loads run ahead of the arithmetic as one stream over all (tile, contraction step) pairs of
-    // the workgroup: the first steps of the next tile are on their way while this one is finished.
-    constexpr int NP = 4;      // chunks per thread and tile, of x and of w
-    uint32_t xoff[NP], woff[NP], xdst[NP], wdst[NP];
-    bool wvalid[NP];
+    // ---- the load stream -----------------------------------------------------------------------
+    // Load instruction i of wave w fills the LDS positions (16-byte units) (w L + i) 64 + lane of a
+    // slot; the lane fetches the chunk that belongs there: x position = row * 8 + (chunk ^ fx(row)),
+    // w position = contraction row * 32 + (chunk ^ fw(row)).  Rows of x beyond M are read from row
+    // M - 1 and feature chunks of w beyond N from chunk 0 (their results are never stored).  The
+    // stream runs over all (tile, slice) pairs of the workgroup: the first slices of the next tile
+    // are on their way while this one is finished.
+    uint32_t xvo[LX], wvo[LW];
     const char* xsrc = nullptr;
     const char* wsrc = nullptr;
     int fetch_tile = logical, fetch_kt = 0;
-    auto aim = [&]() __attribute__((always_inline)) {      // point the loads at the first step of fetch_tile
+    const int ksteps = p.K / KS;
+    auto aim = [&]() __attribute__((always_inline)) {
         int m0, n0;
         tile_origin(fetch_tile, m0, n0);
 #pragma unroll
-        for (int i = 0; i < NP; ++i) {
-            const int idx = tid + i * (kWaves * 64);
-            const int row = min(m0 + (idx >> 3), p.M - 1) - m0;
-            xoff[i] = ((uint32_t)row * (uint32_t)p.K + (uint32_t)(idx & 7) * 8u) * 2u;
-            wvalid[i] = n0 + (idx & 31) * 8 < p.N;
+        for (int i = 0; i < LX; ++i) {
+            const int pos = (wave * LX + i) * 64 + lane;
+            const int row = pos / CPRX;
+            const int c = (pos % CPRX) ^ ((row >> 1) & 7);
+            const int grow = min(m0 + row, p.M - 1) - m0;       // rows beyond M: never stored
+            xvo[i] = ((uint32_t)grow * (uint32_t)p.K + (uint32_t)c * 8u) * 2u;
+        }
+#pragma unroll
+        for (int i = 0; i < LW; ++i) {
+            const int pos = (wave * LW + i) * 64 + lane;
+            const int krow = pos >> 5;
+            int c = (pos & 31) ^ ((krow & 3) << 2);
+            if (n0 + c * 8 >= p.N) c = 0;                        // features beyond N: never stored
+            wvo[i] = ((uint32_t)krow * (uint32_t)p.N + (uint32_t)c * 8u) * 2u;
         }
         xsrc = reinterpret_cast<const char*>(p.x + (int64_t)m0 * p.K);
         wsrc = reinterpret_cast<const char*>(p.w + n0);
     };
+    const uint32_t xs_lds = (uint32_t)(uintptr_t)(FA_LDS void*)xs + (uint32_t)(wave * LX) * 1024u;
+    const uint32_t ws_lds = (uint32_t)(uintptr_t)(FA_LDS void*)ws + (uint32_t)(wave * LW) * 1024u;
+    // The LX + LW loads of a step are issued in two parts, one sub-step apart: 64 KB per step and
+    // compute unit keep the texture path busy for half the step, and a wave that issues all its
+    // loads at once waits at the issue port while the queue drains (measured: +3.5 % for two
+    // parts; four parts, one per sub-step, lose that again because the last ones are issued too
+    // late to land before the step ends).
+    constexpr int NP = 2;
+    constexpr int LPP = (LX + LW) / NP;              // loads per part
+    static_assert((LX + LW) % NP == 0 && NP <= NSUB, "whole loads per part, at most one part per sub-step");
+    auto issue_part = [&](int slot, auto part_c) __attribute__((always_inline)) {
+        constexpr int PART = decltype(part_c)::value;
 #pragma unroll
-    for (int i = 0; i < NP; ++i) {
-        const int idx = tid + i * (kWaves * 64);
-        xdst[i] = (uint32_t)((idx >> 3) * kXStr + (idx & 7) * 8);
-        woff[i] = ((uint32_t)(idx >> 5) * (uint32_t)p.N + (uint32_t)(idx & 31) * 8u) * 2u;
-        wdst[i] = (uint32_t)((idx >> 5) * kWStr + (idx & 31) * 8);
-    }
-    aim();
-    const int ksteps = p.K / kTileK;
-    // two sets of staging registers: a step's data is fetched two steps before it is consumed
-    u32x4 xreg[2][NP], wreg[2][NP];
-    auto fetch = [&](auto set_c) __attribute__((always_inline)) {
-        constexpr int SET = decltype(set_c)::value;
-#pragma unroll
-        for (int i = 0; i < NP; ++i) xreg[SET][i] = *reinterpret_cast<const u32x4*>(xsrc + xoff[i]);
-#pragma unroll
-        for (int i = 0; i < NP; ++i) {
-            wreg[SET][i] = u32x4{0u, 0u, 0u, 0u};
-            if (wvalid[i]) wreg[SET][i] = *reinterpret_cast<const u32x4*>(wsrc + woff[i]);
+        for (int j = PART * LPP; j < (PART + 1) * LPP; ++j) {
+            if (j < LX)
+                dma16(xs_lds + (uint32_t)(slot * XSLOT * 2 + j * 1024), xsrc, xvo[j]);
+            else
+                dma16(ws_lds + (uint32_t)(slot * WSLOT * 2 + (j - LX) * 1024), wsrc, wvo[j - LX]);
         }
-        xsrc += kTileK * 2;
-        wsrc += (int64_t)kTileK * p.N * 2;
-        if (++fetch_kt == ksteps) {
-            fetch_kt = 0;
-            fetch_tile += p.total_wgs;
-            if (fetch_tile < p.total_tiles) aim();
+        if constexpr (PART == NP - 1) {
+            xsrc += KS * 2;
+            wsrc += (int64_t)KS * p.N * 2;
+            if (++fetch_kt == ksteps) {
+                fetch_kt = 0;
+                fetch_tile += p.total_wgs;
+                if (fetch_tile < p.total_tiles) aim();
+            }
         }
     };
-    auto stash = [&](auto set_c, int stage) __attribute__((always_inline)) {
-        constexpr int SET = decltype(set_c)::value;
-#pragma unroll
-        for (int i = 0; i < NP; ++i) *reinterpret_cast<u32x4*>(xs + stage * kXTile + xdst[i]) = xreg[SET][i];
-#pragma unroll
-        for (int i = 0; i < NP; ++i) *reinterpret_cast<u32x4*>(ws + stage * kWTile + wdst[i]) = wreg[SET][i];
+    auto issue = [&](int slot) __attribute__((always_inline)) {
+        issue_part(slot, std::integral_constant<int, 0>{});
+        issue_part(slot, std::integral_constant<int, 1>{});
     };
 
     floatx16 acc[4][2];
@@ -163,17 +184,31 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[nt][mt][r] = 0.f;
 
-    // per-lane parts of the operand addresses
-    // B operand (x): row wm 64 + mt 32 + ln, contraction chunk 2 s + g
-    const _Float16* const xop_base = xs + (wm * 64 + ln) * kXStr + 8 * g;
+    // ---- per-lane parts of the operand addresses (halves inside a slot) ---------------------------
+    // B operand (x): row wm 64 + mt 32 + ln, logical chunk 2 s + g
+    int xrd[NSUB];
+    {
+        const int r0 = wm * 64 + ln;
+        const int fx = (ln >> 1) & 7;      // wm 64 and mt 32 do not reach these bits
+#pragma unroll
+        for (int s = 0; s < NSUB; ++s) xrd[s] = (r0 * CPRX + ((2 * s + g) ^ fx)) * 8;
+    }
     // A operand (w^T), transpose read: lane s16 of a 16-lane group points at contraction row
     // 8 g + s16 / 4 (+ 4 for the second read), features 4 (s16 % 4) ... of the 16 that start at
-    // 16 * ((lane / 16) % 2); feature block nt adds 32.  Lane j of the group receives four
-    // consecutive contraction rows of feature j: slot (g, i) of the operand is contraction index
-    // 16 s + 8 g + i, the order in which the 16-byte read of x delivers them.
-    const int s16 = lane & 15;
-    const _Float16* const wop_base = ws + (8 * g + (s16 >> 2)) * kWStr + wn * 128 + 16 * ((lane >> 4) & 1) +
-                                     4 * (s16 & 3);
+    // 16 * ((lane / 16) % 2) of feature block nt; lane j of the group receives four consecutive
+    // contraction rows of feature j: slot (g, i) of the operand is contraction index 16 s + 8 g + i,
+    // the order in which the 16-byte read of x delivers them.
+    int wrd[4];
+    {
+        const int s16 = lane & 15;
+        const int kk = (s16 >> 2) & 3;
+        const int krow = 8 * g + (s16 >> 2);
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            const int c = wn * 16 + ((nt ^ kk) << 2) + 2 * ((lane >> 4) & 1) + ((s16 & 3) >> 1);
+            wrd[nt] = krow * kTileN + c * 8 + 4 * (s16 & 1);
+        }
+    }
 
     // ---- end of a tile: bias, rotation, one rounding, 8-byte stores; the accumulators start over ---
     // acc[nt][mt][r]: row m = m0 + wm 64 + mt 32 + ln, feature n = n0 + wn 128 + nt 32 + 8 (r / 4) + 4 g + r % 4.
@@ -259,63 +294,103 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
                 for (int r = 0; r < 16; ++r) acc[nt][mt][r] = 0.f;
     };
 
-    // Two LDS stages, two register sets.  Step t of the workgroup's stream consumes its data from LDS
-    // stage t % 2; the loads of step t + 2 are sent off at its start into register set t % 2, and at
-    // its end the data of step t + 1 (requested one step earlier) moves from the other set to the
-    // other stage, which everybody finished reading before the barrier that ended step t - 1.
     const int my_tiles = (p.total_tiles - logical + p.total_wgs - 1) / p.total_wgs;
     const int total_steps = my_tiles * ksteps;
     int tile = logical, kt = 0;
-    auto step = [&](int t, auto par_c) __attribute__((always_inline)) {
-        constexpr int PAR = decltype(par_c)::value;
-        // (at the last step of a tile the loads are sent off behind the epilogue instead, so that no
-        // staging register is live while the epilogue needs registers of its own)
-        const bool last = kt + 1 == ksteps;
-        if (!last && t + 2 < total_steps) fetch(std::integral_constant<int, PAR>{});
-        const _Float16* const xb = xop_base + PAR * kXTile;
-        const _Float16* const wb = wop_base + PAR * kWTile;
+
+    // Operand registers, two sets: the reads of a sub-step are issued before the matrix
+    // instructions of the sub-step before it.
+    half8 wop[2][4], xop[2][2];
+    auto load_ops = [&](auto set_c, int slot, int s) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_c)::value;
+        const _Float16* const xb = xs + slot * XSLOT;
+        const _Float16* const wb = ws + slot * WSLOT;
 #pragma unroll
-        for (int s = 0; s < kTileK / 16; ++s) {
-            half8 wop[4], xop[2];
-#pragma unroll
-            for (int nt = 0; nt < 4; ++nt) {
-                const _Float16* p0 = wb + (16 * s) * kWStr + nt * 32;
-                const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS short4v*)(p0));
-                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS short4v*)(p0 + 4 * kWStr));
-                const short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                wop[nt] = __builtin_bit_cast(half8, both);
-            }
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
-                xop[mt] = *reinterpret_cast<const half8*>(xb + mt * 32 * kXStr + s * 16);
-#pragma unroll
-            for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-                for (int mt = 0; mt < 2; ++mt) {
-                    if constexpr (BF)
-                        acc[nt][mt] = bf16::mfma32(wop[nt], xop[mt], acc[nt][mt]);
-                    else
-                        acc[nt][mt] = mfma32(wop[nt], xop[mt], acc[nt][mt]);
-                }
+        for (int nt = 0; nt < 4; ++nt) {
+            const _Float16* p0 = wb + wrd[nt] + (16 * s) * kTileN;
+            const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS short4v*)(p0));
+            const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS short4v*)(p0 + 4 * kTileN));
+            const short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            wop[SET][nt] = __builtin_bit_cast(half8, both);
         }
-        if (t + 1 < total_steps) stash(std::integral_constant<int, 1 - PAR>{}, 1 - PAR);
-        __syncthreads();
-        if (last) {
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+            xop[SET][mt] = *reinterpret_cast<const half8*>(xb + xrd[s] + mt * 32 * CPRX * 8);
+    };
+    auto multiply = [&](auto set_c) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_c)::value;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+                if constexpr (BF)
+                    acc[nt][mt] = bf16::mfma32(wop[SET][nt], xop[SET][mt], acc[nt][mt]);
+                else
+                    acc[nt][mt] = mfma32(wop[SET][nt], xop[SET][mt], acc[nt][mt]);
+            }
+    };
+    using set0 = std::integral_constant<int, 0>;
+    using set1 = std::integral_constant<int, 1>;
+
+    // Step u reads slot u % 2 while the loads of step u + 1 fill the other one.  One barrier per
+    // step, placed before the matrix instructions of the step's last sub-step: by then every wave
+    // has the operands of that sub-step in registers, so the slot is free for the loads of step
+    // u + 2, and the data of step u + 1 (each wave has waited for its own part) are visible to
+    // everybody, so the operands of its first sub-step are requested before the last matrix
+    // instructions of step u are issued.  The matrix pipe never waits for LDS at a step boundary.
+    static_assert(NSLOT == 2, "the waits below assume that only the next step's loads are in flight");
+    aim();
+    issue(0);
+    if (total_steps > 1) {
+        issue(1);
+        wait_loads<LX + LW>();      // loads complete in order: all but the second step's have landed
+    } else {
+        wait_loads<0>();
+    }
+    ring_barrier();
+    load_ops(set0{}, 0, 0);
+
+    bool pending = false;      // the second part of the loads into the previous step's slot is still to be issued
+    auto step = [&](int u, auto slot_c) __attribute__((always_inline)) {
+        constexpr int SLOT = decltype(slot_c)::value;
+        constexpr int PREV = (SLOT + NSLOT - 1) % NSLOT;
+        // NSUB is even: sub-step s uses register set s % 2, the next step starts with set 0 again
+        auto substep = [&](auto s_c) __attribute__((always_inline)) {
+            constexpr int S = decltype(s_c)::value;
+            load_ops(std::integral_constant<int, (S + 1) & 1>{}, SLOT, S + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (S + 1 < NP) {
+                if (pending) issue_part(PREV, std::integral_constant<int, S + 1>{});
+            }
+            multiply(std::integral_constant<int, S & 1>{});
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        static_assert(NSUB == 4, "three sub-steps before the barrier, one behind it");
+        substep(std::integral_constant<int, 0>{});
+        substep(std::integral_constant<int, 1>{});
+        substep(std::integral_constant<int, 2>{});
+        // this wave's loads of step u + 1 have landed (the stores of an epilogue are waited for
+        // with them), its reads of this step's slot have all returned
+        wait_loads<0>();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        ring_barrier();
+        pending = u + NSLOT < total_steps;
+        if (pending) issue_part(SLOT, std::integral_constant<int, 0>{});
+        if (u + 1 < total_steps) load_ops(set0{}, (SLOT + 1) % NSLOT, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(set1{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (kt + 1 == ksteps) {
             finish_tile(tile);
             kt = 0;
             tile += p.total_wgs;
-            if (t + 2 < total_steps) fetch(std::integral_constant<int, PAR>{});
         } else {
             ++kt;
         }
     };
-    fetch(std::integral_constant<int, 0>{});
-    stash(std::integral_constant<int, 0>{}, 0);
-    if (total_steps > 1) fetch(std::integral_constant<int, 1>{});
-    __syncthreads();
-    for (int t = 0; t < total_steps; t += 2) {
-        step(t, std::integral_constant<int, 0>{});
-        if (t + 1 < total_steps) step(t + 1, std::integral_constant<int, 1>{});
+    for (int u = 0; u < total_steps; u += NSLOT) {
+        step(u, std::integral_constant<int, 0>{});
+        if (u + 1 < total_steps) step(u + 1, std::integral_constant<int, 1>{});
     }
 }
 
