@@ -36,6 +36,8 @@ def _close(got, want, atol=2e-3, rtol=1e-3):
     (2, 129, 256, 6, 32),        # head_dim 32
     (1, 1000, 512, 4, 128),      # head_dim 128
     (4, 512, 1024, 16, 64),      # eight row tiles x twelve feature tiles
+    (1, 8000, 192, 16, 64),      # 384 tiles on 256 workgroups: a second tile behind the first, three slices per tile
+    (2, 5000, 64, 8, 128),       # 480 tiles of one slice each: every step ends a tile
 ])
 @pytest.mark.parametrize("mode", ["plain", "bias", "rope", "bias+rope"])
 def test_projection_matches_the_oracle(gpu, B, L, Fin, R, H, mode):
