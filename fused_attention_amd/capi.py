@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libfused_attn_gfx950.so")
 
 # every symbol include/fused_attn.h declares
 EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_strided", "fa_fwd_plan", "fa_fwd_query", "fa_strerror", "fa_fwd_timed",
-           "fa_qkv_proj")
+           "fa_qkv_proj", "fa_qkv_proj_plan")
 FLAG_CAUSAL = 1
 FLAG_BF16 = 2
 
@@ -52,6 +52,8 @@ def load_library():
     lib.fa_fwd_timed.restype = ctypes.c_int
     lib.fa_qkv_proj.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, vp, ctypes.c_int, vp]
     lib.fa_qkv_proj.restype = ctypes.c_int
+    lib.fa_qkv_proj_plan.argtypes = [i64, i64, i64, i64, i64, ctypes.POINTER(ctypes.c_int)]
+    lib.fa_qkv_proj_plan.restype = ctypes.c_int
     lib.fa_fwd_plan.argtypes = [i64, i64, i64, i64, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int)]
     lib.fa_fwd_plan.restype = ctypes.c_int
     lib.fa_fwd_query.argtypes = [i64]
@@ -76,6 +78,14 @@ def launch_plan(B, R, L, H, causal=False, has_mask=False):
     out = (ctypes.c_int * 6)()
     _check(load_library().fa_fwd_plan(B, R, L, H, FLAG_CAUSAL if causal else 0, 1 if has_mask else 0, out))
     keys = ("waves", "rows_per_wave", "workgroups", "working", "per_head", "heads_per_xcd")
+    return dict(zip(keys, out))
+
+
+def projection_plan(B, L, F_in, R, H):
+    """What fa_qkv_proj_plan reports for a problem, as a dict.  Needs no GPU."""
+    out = (ctypes.c_int * 4)()
+    _check(load_library().fa_qkv_proj_plan(B, L, F_in, R, H, out))
+    keys = ("workgroups", "working", "tiles", "tiles_n")
     return dict(zip(keys, out))
 
 

@@ -452,6 +452,19 @@ hipError_t launch_qkv(const fa::qkv::Params& p, hipStream_t stream) {
                            dim3(kQkvThreads), args, kQkvLds, stream);
 }
 
+// Tiles and grid of the projection kernel for an M x N output.
+int qkv_geometry(int64_t M, int64_t N, fa::qkv::Params* p) {
+    constexpr int64_t kMaxInt = 0x7fffffff;
+    const int64_t tiles_m = ceil_div(M, fa::qkv::kTileM);
+    p->tiles_n = (int)ceil_div(N, fa::qkv::kTileN);
+    if (tiles_m * p->tiles_n > kMaxInt - 8) return FA_ERR_TOO_LARGE;
+    p->total_tiles = (int)(tiles_m * p->tiles_n);
+    // a resident grid, one workgroup per compute unit, each walking through its share of the tiles
+    p->total_wgs = p->total_tiles < kNumCu ? p->total_tiles : kNumCu;
+    p->wgs_per_xcd = (int)ceil_div(p->total_wgs, fa::kNumXcd);
+    return FA_OK;
+}
+
 template <bool BF>
 hipError_t dispatch_qkv(int64_t rope_head_dim, const fa::qkv::Params& p, hipStream_t stream) {
     switch (rope_head_dim) {
@@ -496,17 +509,31 @@ int fa_qkv_proj(const void* x, const void* w, const void* bias, void* qkv, int64
     p.N = (int)(3 * F);
     p.F = (int)F;
     p.L = (int)L;
-    const int64_t tiles_m = ceil_div(B * L, fa::qkv::kTileM);
-    p.tiles_n = (int)ceil_div(3 * F, fa::qkv::kTileN);
-    if (tiles_m * p.tiles_n > kMaxInt - 8) return FA_ERR_TOO_LARGE;
-    p.total_tiles = (int)(tiles_m * p.tiles_n);
-    // a resident grid, one workgroup per compute unit, each walking through its share of the tiles
-    p.total_wgs = p.total_tiles < kNumCu ? p.total_tiles : kNumCu;
-    p.wgs_per_xcd = (int)ceil_div(p.total_wgs, fa::kNumXcd);
+    const int rc = qkv_geometry(B * L, 3 * F, &p);
+    if (rc != FA_OK) return rc;
     const int64_t hr = rope_cos != nullptr ? H : 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const hipError_t e = (flags & FA_FLAG_BF16) != 0 ? dispatch_qkv<true>(hr, p, s) : dispatch_qkv<false>(hr, p, s);
     return static_cast<int>(e);
+}
+
+int fa_qkv_proj_plan(int64_t B, int64_t L, int64_t F_in, int64_t R, int64_t H, int* plan) {
+    if (plan == nullptr) return FA_ERR_NULL_POINTER;
+    if (!fa_fwd_query(H)) return FA_ERR_BAD_HEAD_DIM;
+    if (B < 1 || L < 1 || R < 1 || F_in < 1) return FA_ERR_BAD_SHAPE;
+    constexpr int64_t kMaxInt = 0x7fffffff;
+    if (B > kMaxInt || L > kMaxInt || R > kMaxInt || B * L > kMaxInt - 2 * fa::qkv::kTileM) return FA_ERR_TOO_LARGE;
+    const int64_t F = R * H;
+    if (F_in % fa::qkv::kTileK != 0 || F % 64 != 0) return FA_ERR_BAD_SHAPE;
+    if (F_in > ((int64_t)1 << 22) || F > ((int64_t)1 << 22)) return FA_ERR_TOO_LARGE;
+    fa::qkv::Params p;
+    const int rc = qkv_geometry(B * L, 3 * F, &p);
+    if (rc != FA_OK) return rc;
+    plan[0] = p.wgs_per_xcd * fa::kNumXcd;
+    plan[1] = p.total_wgs;
+    plan[2] = p.total_tiles;
+    plan[3] = p.tiles_n;
+    return FA_OK;
 }
 
 }  // extern "C"

@@ -160,6 +160,14 @@ int fa_qkv_proj(const void* x, const void* w, const void* bias, void* qkv,
                 int64_t B, int64_t L, int64_t F_in, int64_t R, int64_t H,
                 const float* rope_cos, const float* rope_sin, int flags, void* stream);
 
+/*
+ * The launch fa_qkv_proj would make for a problem, without making it (no GPU is touched): for
+ * tests of the launcher.  Fills plan[0..3] with: workgroups launched; workgroups that do work (a
+ * resident grid: workgroup w of them takes the tiles w, w + working, ...); output tiles of 256 x 256
+ * (row tiles times feature tiles); feature tiles.  No counterpart in the reference (see fa_qkv_proj).
+ */
+int fa_qkv_proj_plan(int64_t B, int64_t L, int64_t F_in, int64_t R, int64_t H, int* plan);
+
 #ifdef __cplusplus
 }
 #endif

@@ -134,6 +134,44 @@ def test_every_launch_plan_covers_every_query_tile_once():
     assert dealt > 10          # the dealt schedule was among the plans
 
 
+def _tiles_of_projection_plan(plan):
+    """Replays how qkv_proj_kernel (qkv_proj_kernel.hpp) turns a workgroup index into output tiles
+    (row tile, feature tile)."""
+    per_xcd = plan["workgroups"] // 8
+    tiles_m = plan["tiles"] // plan["tiles_n"]
+    band_of = 4
+    tiles = []
+    for wg in range(plan["workgroups"]):
+        logical = (wg % 8) * per_xcd + wg // 8
+        if logical >= plan["working"]:
+            continue
+        for tile in range(logical, plan["tiles"], plan["working"]):
+            band, in_band = divmod(tile, band_of * plan["tiles_n"])
+            band_rows = min(band_of, tiles_m - band * band_of)
+            row_tile = band * band_of + in_band % band_rows
+            col_tile = in_band // band_rows
+            assert row_tile < tiles_m and col_tile < plan["tiles_n"]
+            tiles.append((row_tile, col_tile))
+    return tiles, tiles_m
+
+
+def test_every_projection_plan_covers_every_output_tile_once():
+    """fa_qkv_proj's grid parameters against the kernel's decoding of them, on the CPU: every
+    256 x 256 output tile exactly once, over shapes with 1 ... 1920 tiles."""
+    shapes = [(4, 2048, 5120, 40, 128), (4, 4096, 1024, 16, 64), (1, 8000, 192, 16, 64), (2, 5000, 64, 8, 128),
+              (1, 64, 64, 1, 64), (1, 257, 192, 3, 64), (1, 16384, 4096, 32, 128), (1, 5400, 64, 16, 64),
+              (3, 2222, 128, 12, 64), (1, 66000, 64, 1, 64), (2, 4096, 64, 11, 64)]
+    for B, L, F_in, R, H in shapes:
+        plan = capi.projection_plan(B, L, F_in, R, H)
+        tiles, tiles_m = _tiles_of_projection_plan(plan)
+        assert plan["tiles"] == -(-B * L // 256) * -(-3 * R * H // 256)
+        assert plan["working"] == min(plan["tiles"], 256) and plan["workgroups"] >= plan["working"]
+        assert len(tiles) == plan["tiles"], (B, L, F_in, R, H, plan)
+        assert set(tiles) == {(r, c) for r in range(tiles_m) for c in range(plan["tiles_n"])}, (B, L, R, H, plan)
+    with pytest.raises(capi.FusedAttnError):
+        capi.projection_plan(1, 64, 100, 1, 64)          # contraction length not a multiple of 64
+
+
 def test_benchmark_workloads_take_the_kernels_the_documentation_names():
     def plan(B, R, L, H, **kw):
         p = capi.launch_plan(B, R, L, H, **kw)

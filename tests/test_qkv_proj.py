@@ -38,6 +38,7 @@ def _close(got, want, atol=2e-3, rtol=1e-3):
     (4, 512, 1024, 16, 64),      # eight row tiles x twelve feature tiles
     (1, 8000, 192, 16, 64),      # 384 tiles on 256 workgroups: a second tile behind the first, three slices per tile
     (2, 5000, 64, 8, 128),       # 480 tiles of one slice each: every step ends a tile
+    (1, 5476, 128, 16, 64),      # 264 tiles: eight workgroups take a second one; the last row tile holds 100 rows
 ])
 @pytest.mark.parametrize("mode", ["plain", "bias", "rope", "bias+rope"])
 def test_projection_matches_the_oracle(gpu, B, L, Fin, R, H, mode):
