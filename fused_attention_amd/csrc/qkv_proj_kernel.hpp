@@ -23,7 +23,8 @@
 // (ds_read_b64_tr_b16), the B operand X^T (16 k x 32 rows m) is a plain 16-byte read of a row of x.
 // In the accumulator a lane then owns one output row m and, per 32 x 32 block, 16 output features
 // n in runs of four: bias and rotation are applied in registers (the partner feature n + H/2 of a
-// rotation sits in the same lane), and a run is stored with one 8-byte store.
+// rotation sits in the same lane); the rounded rows then pass through a small per-wave LDS tile
+// and leave as whole 256-byte row segments with streaming stores.
 //
 // A wave owns 64 rows x 128 features (4 x 2 blocks of 32 x 32, 128 accumulator registers); its
 // 128 features are whole heads for every head_dim up to 128.
@@ -40,7 +41,9 @@ constexpr int kTileK = 64;    // contraction steps per slice (one ring slot)
 constexpr int kWaves = 8;
 constexpr int kBand = 4;      // row tiles per band of the tile order
 constexpr int kSlots = 2;     // ring slots: one is read while the other is filled
-constexpr int kLdsBytes = kSlots * (kTileM + kTileN) * kTileK * (int)sizeof(_Float16);   // 128 KB
+constexpr int kRingHalves = kSlots * (kTileM + kTileN) * kTileK;                           // 128 KB
+constexpr int kStageHalves = 16 * 128;      // per wave: 16 output rows of the wave's 128 features (4 KB)
+constexpr int kLdsBytes = (kRingHalves + kWaves * kStageHalves) * (int)sizeof(_Float16);   // 160 KB
 
 struct Params {
     const _Float16* x;       // [M, K]
@@ -90,6 +93,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
     const int ln = lane & 31;
     const int wm = wave >> 1;
     const int wn = wave & 1;
+    _Float16* const stage = smem + kRingHalves + wave * kStageHalves;     // this wave's output staging tile
 
     // A resident grid: workgroup `logical` takes the tiles logical, logical + G, logical + 2 G, ...
     // Workgroups are dealt round-robin to the XCDs, so they are renumbered first: one XCD (one L2)
@@ -210,7 +214,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
         }
     }
 
-    // ---- end of a tile: bias, rotation, one rounding, 8-byte stores; the accumulators start over ---
+    // ---- end of a tile: bias, rotation, one rounding, whole-row stores; the accumulators start over ---
     // acc[nt][mt][r]: row m = m0 + wm 64 + mt 32 + ln, feature n = n0 + wn 128 + nt 32 + 8 (r / 4) + 4 g + r % 4.
     // The accumulators are only read here (results are formed in temporaries): modifying them in
     // place inside the step loop makes the compiler carry a second copy of all of them.
@@ -228,17 +232,29 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
             }
             return v;
         };
-        auto store_run = [&](floatx4 v, int m, int n) __attribute__((always_inline)) {
-            if (m < p.M && n < p.N) {
+        // The results leave through a private LDS tile of 16 rows x 128 features per wave, so that
+        // every store instruction writes whole rows (16 lanes x 16 bytes = the wave's 256 bytes of a
+        // row) as streaming stores, instead of 8 bytes into each of 32 rows.  A lane holds one row
+        // of a 32-row block: the block goes out in two halves of 16 rows, the lanes of the other half
+        // sitting the pass out.  Chunk c (16 bytes) of stage row r sits at c ^ r: the 16
+        // rows of one chunk column and the 16 chunks of one row both cover all banks.
+        auto store_run = [&](floatx4 v, int nt, int r4) __attribute__((always_inline)) {
+            {
                 u16x4 hv;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) hv[e] = BF ? bf16::float_to_elem(v[e]) : float_to_elem(v[e]);
-                *reinterpret_cast<u32x2*>(p.out + (int64_t)m * p.N + n) = __builtin_bit_cast(u32x2, hv);
+                // (the row index is made opaque per run: otherwise the 16 swizzled addresses of a row
+                // are all computed ahead and held in registers through the whole epilogue)
+                int r = ln & 15;
+                asm volatile("" : "+v"(r));
+                *reinterpret_cast<u32x2*>(stage + r * 128 + (((nt * 4 + r4) ^ r) * 8) + 4 * g) = __builtin_bit_cast(u32x2, hv);
             }
         };
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
+        for (int mh = 0; mh < 4; ++mh) {
+            const int mt = mh >> 1, half = mh & 1;
             const int m = m0 + wm * 64 + mt * 32 + ln;
+            if ((ln >> 4) == half) {        // the other half of the lanes sits this pass out (no table or bias loads)
             if constexpr (HR > 0) {
                 // rotate-half: within a head, feature i < HR / 2 pairs with feature i + HR / 2:
                 //   out[i] = y[i] cos_i - y[i + HR/2] sin_i,  out[i + HR/2] = y[i + HR/2] cos_i + y[i] sin_i
@@ -271,8 +287,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
                         a = ra;
                         b = rb;
                     }
-                    store_run(a, m, n_a);
-                    store_run(b, m, n_b);
+                    store_run(a, nt_a, r4_a);
+                    store_run(b, nt_b, r4_b);
                     // one pair at a time: all table loads at once would not fit in the registers
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -282,9 +298,23 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
 #pragma unroll
                     for (int r4 = 0; r4 < 4; ++r4) {
                         const int n = nw + nt * 32 + 8 * r4 + 4 * g;
-                        store_run(biased(nt, mt, r4, n), m, n);
+                        store_run(biased(nt, mt, r4, n), nt, r4);
                     }
             }
+            }
+            // LDS operations of one wave complete in order; the waits keep the compiler from moving
+            // the reads above the writes (and the next half's writes above these reads)
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = 4 * i + (lane >> 4), ch = lane & 15;
+                const u32x4 w = *reinterpret_cast<const u32x4*>(stage + r * 128 + ((ch ^ r) * 8));
+                const int mr = m0 + wm * 64 + mt * 32 + half * 16 + r;
+                const int n = nw + ch * 8;
+                if (mr < p.M && n < p.N)
+                    __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(p.out + (int64_t)mr * p.N + n));
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         }
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt)
@@ -376,14 +406,19 @@ __global__ __launch_bounds__(kWaves * 64, 2) void qkv_proj_kernel(const Params p
         ring_barrier();
         pending = u + NSLOT < total_steps;
         if (pending) issue_part(SLOT, std::integral_constant<int, 0>{});
-        if (u + 1 < total_steps) load_ops(set0{}, (SLOT + 1) % NSLOT, 0);
+        // (at the end of a tile the operands of the next step are requested behind the epilogue, which
+        // needs the registers)
+        const bool last = kt + 1 == ksteps;
+        if (u + 1 < total_steps && !last) load_ops(set0{}, (SLOT + 1) % NSLOT, 0);
         __builtin_amdgcn_sched_barrier(0);
         multiply(set1{});
         __builtin_amdgcn_sched_barrier(0);
-        if (kt + 1 == ksteps) {
+        if (last) {
             finish_tile(tile);
             kt = 0;
             tile += p.total_wgs;
+            __builtin_amdgcn_sched_barrier(0);
+            if (u + 1 < total_steps) load_ops(set0{}, (SLOT + 1) % NSLOT, 0);
         } else {
             ++kt;
         }
