@@ -175,6 +175,7 @@ def projection_workload(name, dev, rope, iters=None):
     flop = 2.0 * w.B * w.L * F * 3 * F
     step()
     torch.cuda.synchronize()
+    profiled_iters = iters
     if iters is None:
         iters = max(20, min(2000, int(0.3 / (flop / 0.9e15))))
     for _ in range(iters):
@@ -186,6 +187,21 @@ def projection_workload(name, dev, rope, iters=None):
     e1.record()
     torch.cuda.synchronize()
     kernel_ms = e0.elapsed_time(e1) / iters
+    # for scale, the vendor library's plain GEMM on the same operands (no bias, no rotation, an
+    # [M, 3F] result), timed the same way; left out of profiled runs (iters given)
+    vendor = None
+    if profiled_iters is None and not rope:
+        x2, o2 = xd.view(w.B * w.L, F), torch.empty(w.B * w.L, 3 * F, dtype=torch.float16, device=dev)
+        for _ in range(iters):
+            torch.matmul(x2, wd, out=o2)
+        e0.record()
+        for _ in range(iters):
+            torch.matmul(x2, wd, out=o2)
+        e1.record()
+        torch.cuda.synchronize()
+        vendor_ms = e0.elapsed_time(e1) / iters
+        vendor = {"what": "torch.matmul (hipBLASLt) on the same x and w", "kernel_ms": vendor_ms,
+                  "tflops": flop / (vendor_ms * 1e-3) / 1e12}
     rows = torch.arange(0, w.L, max(1, w.L // 64))
     want = qkv_projection(x[:1, rows], wt, None, w.R, w.H, *((tables[0][rows], tables[1][rows]) if rope else (None, None)))
     got = out[:1, rows.to(dev)].float().cpu()
@@ -202,6 +218,7 @@ def projection_workload(name, dev, rope, iters=None):
         "bytes_algorithmic": (w.B * w.L * F + F * 3 * F + w.B * w.L * 3 * F) * 2,
         "traffic": None if rope else MEASURED_TRAFFIC.get("qkv_proj_" + name, (None, None))[0],
         "traffic_source": None if rope else MEASURED_TRAFFIC.get("qkv_proj_" + name, (None, None))[1],
+        "vendor_gemm": vendor,
     }
 
 
