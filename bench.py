@@ -36,6 +36,7 @@ PEAK_TFLOPS_FP16 = 2500.0   # MI355X dense fp16 MFMA, published
 MEASURED_TRAFFIC = {
     "c3": (134.4e6, "profiles/fwd_kernel_pingpong_c3.md"),
     "c4": (806.5e6, "profiles/fwd_kernel_pingpong_c4.md"),
+    "readme": (335.7e6, "profiles/fwd_kernel_pingpong_readme.md"),
     "qkv_proj_c3": (269.4e6, "profiles/qkv_proj_kernel_c3.md"),
     "qkv_proj_readme": (2181.4e6, "profiles/qkv_proj_kernel_readme.md"),
 }
