@@ -304,3 +304,18 @@ def test_ctypes_wrapper_checks_tensors_before_any_address_reaches_the_library(mo
     both("torch.Tensor", exc=TypeError, k=[1, 2, 3])
     with pytest.raises(ValueError, match="shape of q"):
         capi.forward(q, q, q, H, out=out[:, :32])
+
+
+def test_bench_refuses_more_than_one_gpu_and_a_machine_without_one():
+    """bench.py measures one GPU; with --gpus 2 it says so and exits, and on a machine without a
+    GPU it fails instead of timing anything else."""
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(REPO, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in (r.stdout + r.stderr)
+    if not torch.cuda.is_available():
+        r = subprocess.run([sys.executable, os.path.join(REPO, "bench.py"), "--steps", "1", "--warmup", "0"],
+                           capture_output=True, text=True)
+        assert r.returncode != 0 and "needs a GPU" in (r.stdout + r.stderr)
+        assert '"metric"' not in r.stdout
