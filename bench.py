@@ -148,6 +148,62 @@ def side_workload(name, dev, check_budget_s):
     return entry
 
 
+def variant_workload(name, dev, variant):
+    """The extensions of the C ABI on a benchmark configuration: 'bf16' (bfloat16 tensors), 'causal',
+    'mask' (an additive fp16 [B, L, L] mask of zeros below and -inf above the diagonal, which gives
+    the causal result).  Kernel time from events on the launch stream around back-to-back launches
+    through capi.forward; flop counts every (query, key) pair the variant attends to; error
+    against the float32 oracle on the first (batch, head) pair."""
+    import torch
+
+    from fused_attention_amd import capi, workloads
+    from oracle import attention, causal_mask
+
+    w = workloads.WORKLOADS[name]
+    q, k, v = workloads.make_inputs(w)
+    dt = torch.bfloat16 if variant == "bf16" else torch.float16
+    q, k, v = q.to(dt), k.to(dt), v.to(dt)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    causal = variant == "causal"
+    mask = None
+    if variant == "mask":
+        mask = torch.full((w.L, w.L), float("-inf")).triu(1).to(torch.float16).expand(w.B, w.L, w.L).contiguous().to(dev)
+    out = torch.empty_like(qd)
+
+    def step():
+        return capi.forward(qd, kd, vd, w.H, out=out, causal=causal, mask=mask)
+
+    step()
+    torch.cuda.synchronize()
+    flop = workloads.flops(w) if variant == "bf16" else 2.0 * w.B * w.R * w.L * (w.L + 1) * w.H
+    iters = max(50, min(3000, int(0.3 / (flop / 0.8e15))))
+    for _ in range(iters):
+        step()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    kernel_ms = e0.elapsed_time(e1) / iters
+    # the first (batch, head) pair as a one-head problem of its own
+    q1, k1, v1 = (t[:1, :, :w.H].float() for t in (q, k, v))
+    ref = attention(q1, k1, v1, w.H, mask=None if variant == "bf16" else causal_mask(1, w.L))
+    got = out[:1, :, :w.H].float().cpu()
+    tflops = flop / (kernel_ms * 1e-3) / 1e12
+    return {
+        "shape": "B=%d R=%d L=%d H=%d %s" % (w.B, w.R, w.L, w.H, variant),
+        "kernel_ms": kernel_ms,
+        "launches_timed": iters,
+        "flop_counted": "4*B*R*L^2*H" if variant == "bf16" else "2*B*R*L*(L+1)*H (pairs at or below the diagonal)",
+        "tflops": tflops,
+        "frac": tflops / PEAK_TFLOPS_FP16,
+        "max_abs_err": (got - ref).abs().max().item(),
+        "finite": bool(torch.isfinite(out.float()).all()),
+        "pairs_checked": 1,
+    }
+
+
 def projection_workload(name, dev, rope, iters=None):
     """The fused QKV projection front end (fa_qkv_proj) at the feature sizes of a benchmark
     configuration: hidden [B, L, R*H] times weight [R*H, 3*R*H] into the packed qkv tensor the
@@ -362,6 +418,8 @@ def main():
         line["workloads"] = {name: side_workload(name, dev, args.check_budget_s)
                              for name in OTHER_WORKLOADS if name != args.workload}
         # the projection front end at the headline's and the reference benchmark's feature sizes
+        for variant in ("bf16", "causal", "mask"):
+            line["workloads"]["c3_" + variant] = variant_workload("c3", dev, variant)
         line["workloads"]["qkv_proj_c3"] = projection_workload("c3", dev, rope=False)
         line["workloads"]["qkv_proj_c3_rotary"] = projection_workload("c3", dev, rope=True)
         line["workloads"]["qkv_proj_readme"] = projection_workload("readme", dev, rope=False)
