@@ -417,9 +417,10 @@ def main():
         torch.cuda.empty_cache()
         line["workloads"] = {name: side_workload(name, dev, args.check_budget_s)
                              for name in OTHER_WORKLOADS if name != args.workload}
-        # the projection front end at the headline's and the reference benchmark's feature sizes
+        # the extensions of the C ABI on the headline configuration
         for variant in ("bf16", "causal", "mask"):
             line["workloads"]["c3_" + variant] = variant_workload("c3", dev, variant)
+        # the projection front end at the headline's and the reference benchmark's feature sizes
         line["workloads"]["qkv_proj_c3"] = projection_workload("c3", dev, rope=False)
         line["workloads"]["qkv_proj_c3_rotary"] = projection_workload("c3", dev, rope=True)
         line["workloads"]["qkv_proj_readme"] = projection_workload("readme", dev, rope=False)
