@@ -9,7 +9,8 @@ pairs.  Counterpart of the reference's benchmark (reference tests/benchmark_fuse
 which prints wall-clock milliseconds of 128 naive and 128 fused launches.
 
 Before the counted warm-up the step is launched for half a second, so that the chip's clock has
-settled ("settle_launches").  With the default workload the line also carries "workloads": kernel
+settled ("settle_launches"); "value_cold" is the same measurement taken before that loop, after
+the --warmup launches only.  With the default workload the line also carries "workloads": kernel
 time, TFLOP/s, roofline fraction and error on a bounded sample for the other configurations and for
 the QKV projection front end.
 
@@ -151,9 +152,9 @@ def side_workload(name, dev, check_budget_s):
 def variant_workload(name, dev, variant):
     """The extensions of the C ABI on a benchmark configuration: 'bf16' (bfloat16 tensors), 'causal',
     'mask' (an additive fp16 [B, L, L] mask of zeros below and -inf above the diagonal, which gives
-    the causal result).  Kernel time from events on the launch stream around back-to-back launches
-    through capi.forward; flop counts every (query, key) pair the variant attends to; error
-    against the float32 oracle on the first (batch, head) pair."""
+    the causal result).  Kernel time from HIP events around back-to-back launches inside the kernel
+    library (fa_fwd_timed_ex), after a settle loop; flop counts every (query, key) pair the variant
+    attends to; error against the float32 oracle on four (batch, head) pairs."""
     import torch
 
     from fused_attention_amd import capi, workloads
@@ -170,26 +171,25 @@ def variant_workload(name, dev, variant):
         mask = torch.full((w.L, w.L), float("-inf")).triu(1).to(torch.float16).expand(w.B, w.L, w.L).contiguous().to(dev)
     out = torch.empty_like(qd)
 
-    def step():
-        return capi.forward(qd, kd, vd, w.H, out=out, causal=causal, mask=mask)
-
-    step()
+    capi.forward(qd, kd, vd, w.H, out=out, causal=causal, mask=mask)
     torch.cuda.synchronize()
     flop = workloads.flops(w) if variant == "bf16" else 2.0 * w.B * w.R * w.L * (w.L + 1) * w.H
-    iters = max(50, min(3000, int(0.3 / (flop / 0.8e15))))
-    for _ in range(iters):
-        step()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        step()
-    e1.record()
-    torch.cuda.synchronize()
-    kernel_ms = e0.elapsed_time(e1) / iters
-    # the first (batch, head) pair as a one-head problem of its own
-    q1, k1, v1 = (t[:1, :, :w.H].float() for t in (q, k, v))
-    ref = attention(q1, k1, v1, w.H, mask=None if variant == "bf16" else causal_mask(1, w.L))
-    got = out[:1, :, :w.H].float().cpu()
+
+    def timed(iters):
+        return capi.forward_timed(qd, kd, vd, w.H, out, iters=iters, causal=causal, mask=mask)
+
+    one = max(timed(3), 1e-3)
+    timed(max(8, int(0.3e3 / one)))                 # settle
+    iters = max(50, min(5000, int(0.3e3 / one)))
+    kernel_ms = timed(iters)
+    # four (batch, head) pairs spread over batches and heads, each as a one-head problem of its own
+    pairs = sorted({(b, h) for b, h in ((0, 0), (w.B - 1, w.R - 1), (w.B // 2, w.R // 3), (w.B // 3, (2 * w.R) // 3))})
+    err = 0.0
+    for b, h in pairs:
+        cols = slice(h * w.H, (h + 1) * w.H)
+        q1, k1, v1 = (t[b:b + 1, :, cols].float() for t in (q, k, v))
+        ref = attention(q1, k1, v1, w.H, mask=None if variant == "bf16" else causal_mask(1, w.L))
+        err = max(err, (out[b:b + 1, :, cols].float().cpu() - ref).abs().max().item())
     tflops = flop / (kernel_ms * 1e-3) / 1e12
     return {
         "shape": "B=%d R=%d L=%d H=%d %s" % (w.B, w.R, w.L, w.H, variant),
@@ -198,9 +198,11 @@ def variant_workload(name, dev, variant):
         "flop_counted": "4*B*R*L^2*H" if variant == "bf16" else "2*B*R*L*(L+1)*H (pairs at or below the diagonal)",
         "tflops": tflops,
         "frac": tflops / PEAK_TFLOPS_FP16,
-        "max_abs_err": (got - ref).abs().max().item(),
+        "max_abs_err": err,
         "finite": bool(torch.isfinite(out.float()).all()),
-        "pairs_checked": 1,
+        "pairs_checked": len(pairs),
+        "traffic": MEASURED_TRAFFIC.get(name + "_" + variant, (None, None))[0],
+        "traffic_source": MEASURED_TRAFFIC.get(name + "_" + variant, (None, None))[1],
     }
 
 
@@ -349,28 +351,24 @@ def main():
         def step():
             return fused_attn.attention_forward(w.H, chunk, qd, kd, vd)
 
-    settle_launches = settle(step, SETTLE_SECONDS)
-    for _ in range(args.warmup):
-        out = step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        out = step()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall / args.steps * 1e3
-
-    # Kernel duration: HIP events on the launch stream around back-to-back launches.
-    if args.causal:
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(args.steps):
-            step()
-        e1.record()
+    def timed_steps():
+        for _ in range(args.warmup):
+            o = step()
         torch.cuda.synchronize()
-        kernel_ms = e0.elapsed_time(e1) / args.steps
-    else:
-        kernel_ms = capi.forward_timed(qd, kd, vd, w.H, out, iters=args.steps)
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            o = step()
+        torch.cuda.synchronize()
+        return o, (time.perf_counter() - t0) / args.steps * 1e3
+
+    # First without the settle loop ("value_cold": what --warmup and --steps alone read, the
+    # figure earlier versions of this script reported as `value`), then after it.
+    out, ms_per_step_cold = timed_steps()
+    settle_launches = settle(step, SETTLE_SECONDS)
+    out, ms_per_step = timed_steps()
+
+    # Kernel duration: HIP events on the launch stream around back-to-back launches, inside the library.
+    kernel_ms = capi.forward_timed(qd, kd, vd, w.H, out, iters=args.steps, causal=args.causal)
 
     # causal: query i attends to i + 1 keys
     flop = 2.0 * w.B * w.R * w.L * (w.L + 1) * w.H if args.causal else workloads.flops(w)
@@ -386,6 +384,8 @@ def main():
         "warmup": args.warmup,
         "settle_launches": settle_launches,
         "ms_per_step": ms_per_step,
+        "value_cold": flop / (ms_per_step_cold * 1e-3) / 1e12,
+        "ms_per_step_cold": ms_per_step_cold,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

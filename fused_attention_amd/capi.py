@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libfused_attn_gfx950.so")
 
 # every symbol include/fused_attn.h declares
 EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_strided", "fa_fwd_plan", "fa_fwd_query", "fa_strerror", "fa_fwd_timed",
-           "fa_qkv_proj", "fa_qkv_proj_plan")
+           "fa_fwd_timed_ex", "fa_qkv_proj", "fa_qkv_proj_plan")
 FLAG_CAUSAL = 1
 FLAG_BF16 = 2
 
@@ -50,6 +50,8 @@ def load_library():
     lib.fa_fwd_strided.restype = ctypes.c_int
     lib.fa_fwd_timed.argtypes = fwd_args + [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
     lib.fa_fwd_timed.restype = ctypes.c_int
+    lib.fa_fwd_timed_ex.argtypes = lib.fa_fwd_strided.argtypes + [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+    lib.fa_fwd_timed_ex.restype = ctypes.c_int
     lib.fa_qkv_proj.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, vp, vp, ctypes.c_int, vp]
     lib.fa_qkv_proj.restype = ctypes.c_int
     lib.fa_qkv_proj_plan.argtypes = [i64, i64, i64, i64, i64, ctypes.POINTER(ctypes.c_int)]
@@ -209,25 +211,25 @@ def forward(q, k, v, head_dim, out=None, mask=None, layout="blf", scale=None, ca
     return (out, lse) if return_lse else out
 
 
-def forward_timed(q, k, v, head_dim, out, iters, mask=None, layout="blf", scale=None):
-    """Average milliseconds per launch over `iters` back-to-back launches (HIP events on the
-    launch stream, measured inside the library).  fp16 only; q, k, v and out share one set of
-    strides (fa_fwd_timed has no output strides of its own)."""
+def forward_timed(q, k, v, head_dim, out, iters, mask=None, layout="blf", scale=None, causal=False):
+    """Average milliseconds per launch over `iters` back-to-back launches of the launch `forward`
+    would make (HIP events on the launch stream, measured inside the library by fa_fwd_timed_ex).
+    Same tensors as `forward` (fp16 or bf16, views allowed); `out` is required."""
     import torch
 
     B, R, L, (sb, sh, sl) = _checked_problem(q, k, v, head_dim, out, mask, layout)
-    if q.dtype != torch.float16:
-        raise TypeError("forward_timed takes float16 tensors, got %s" % q.dtype)
-    if out is None or _strides(out, head_dim, layout, "out") != (sb, sh, sl):
-        raise ValueError("forward_timed needs an `out` tensor with the strides of q")
+    if out is None:
+        raise ValueError("forward_timed needs an `out` tensor")
+    flags = (FLAG_CAUSAL if causal else 0) | (FLAG_BF16 if q.dtype == torch.bfloat16 else 0)
+    ob, oh, ol = _strides(out, head_dim, layout, "out")
     if scale is None:
         scale = 1.0 / math.sqrt(head_dim)
     ms = ctypes.c_float(0.0)
     with torch.cuda.device(q.device):
-        status = load_library().fa_fwd_timed(
+        status = load_library().fa_fwd_timed_ex(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr() if mask is not None else None,
-            out.data_ptr(), B, R, L, head_dim, sb, sh, sl, scale, _current_stream(q) or None,
-            int(iters), ctypes.byref(ms))
+            out.data_ptr(), None, B, R, L, head_dim, sb, sh, sl, ob, oh, ol, scale, flags,
+            _current_stream(q) or None, int(iters), ctypes.byref(ms))
     _check(status)
     return float(ms.value)
 
@@ -247,8 +249,17 @@ def qkv_project(x, w, num_heads, head_dim, bias=None, rope=None, out=None):
         raise TypeError("x must be float16 or bfloat16, got %s" % x.dtype)
     if x.dim() != 3 or w.dim() != 2:
         raise ValueError("x must be [B, L, F_in] and w [F_in, 3 F]")
+    if int(head_dim) != head_dim or head_dim not in (16, 32, 64, 128):
+        raise ValueError("head_dim must be 16, 32, 64 or 128, got %r" % (head_dim,))
+    if int(num_heads) != num_heads or num_heads < 1:
+        raise ValueError("num_heads must be a positive integer, got %r" % (num_heads,))
     B, L, f_in = x.shape
     F = num_heads * head_dim
+    if F % 64 != 0:
+        raise ValueError("num_heads * head_dim (%d) must be a multiple of 64: the three slices of the packed "
+                         "output start on 64-feature boundaries" % F)
+    if f_in % 64 != 0:
+        raise ValueError("F_in (%d) must be a multiple of 64: the contraction is walked in steps of 64" % f_in)
     if tuple(w.shape) != (f_in, 3 * F):
         raise ValueError("w must have shape [F_in, 3 * num_heads * head_dim] = [%d, %d], got %s"
                          % (f_in, 3 * F, tuple(w.shape)))
@@ -260,6 +271,8 @@ def qkv_project(x, w, num_heads, head_dim, bias=None, rope=None, out=None):
         raise ValueError("out must have shape [%d, %d, 3, %d], got %s" % (B, L, F, tuple(out.shape)))
     tables = (None, None)
     if rope is not None:
+        if isinstance(rope, torch.Tensor) or not isinstance(rope, (tuple, list)) or len(rope) != 2:
+            raise ValueError("rope must be a pair (cos, sin) of float32 [L, head_dim / 2] tensors")
         tables = tuple(rope)
         for name, t in zip(("rope cos", "rope sin"), tables):
             if not isinstance(t, torch.Tensor) or t.dtype != torch.float32 or tuple(t.shape) != (L, head_dim // 2):

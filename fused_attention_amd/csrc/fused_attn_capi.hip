@@ -271,8 +271,9 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     if (L > kMaxInt - 4096 || B > kMaxInt || R > kMaxInt || B * R > kMaxInt) return FA_ERR_TOO_LARGE;
     // the tile loaders keep 32-bit byte offsets inside a 64-key tile
     if (stride_l > ((int64_t)1 << 24)) return FA_ERR_TOO_LARGE;
+    // (the eight-wave kernel keeps 32-bit byte offsets inside the 64 mask rows of a wave)
     *shape = pick_shape(B, R, L, H, mask != nullptr,
-                        (L % 8) == 0 && (reinterpret_cast<uintptr_t>(mask) & 15u) == 0, causal);
+                        (L % 8) == 0 && L <= ((int64_t)1 << 24) && (reinterpret_cast<uintptr_t>(mask) & 15u) == 0, causal);
     const int64_t bq = shape->rows();
     int64_t n_qtiles = (L + bq - 1) / bq;
     int64_t total = 0;
@@ -402,9 +403,10 @@ int fa_fwd(const void* q, const void* k, const void* v, const void* mask, void* 
                      stream);
 }
 
-int fa_fwd_timed(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,
-                 int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h,
-                 int64_t stride_l, float scale, void* stream, int iters, float* ms_per_launch) {
+int fa_fwd_timed_ex(const void* q, const void* k, const void* v, const void* mask, void* out, void* lse,
+                    int64_t B, int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h,
+                    int64_t stride_l, int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_l,
+                    float scale, int flags, void* stream, int iters, float* ms_per_launch) {
     if (ms_per_launch == nullptr) return FA_ERR_NULL_POINTER;
     if (iters < 1) return FA_ERR_BAD_SHAPE;
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -420,7 +422,8 @@ int fa_fwd_timed(const void* q, const void* k, const void* v, const void* mask, 
     e = hipEventRecord(e0, s);
     if (e != hipSuccess) rc = static_cast<int>(e);
     for (int i = 0; i < iters && rc == FA_OK; ++i)
-        rc = fa_fwd(q, k, v, mask, out, B, R, L, H, stride_b, stride_h, stride_l, scale, stream);
+        rc = fa_fwd_strided(q, k, v, mask, out, lse, B, R, L, H, stride_b, stride_h, stride_l, out_stride_b,
+                            out_stride_h, out_stride_l, scale, flags, stream);
     if (rc == FA_OK) {
         e = hipEventRecord(e1, s);
         if (e == hipSuccess) e = hipEventSynchronize(e1);
@@ -434,6 +437,13 @@ int fa_fwd_timed(const void* q, const void* k, const void* v, const void* mask, 
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     return rc;
+}
+
+int fa_fwd_timed(const void* q, const void* k, const void* v, const void* mask, void* out, int64_t B,
+                 int64_t R, int64_t L, int64_t H, int64_t stride_b, int64_t stride_h,
+                 int64_t stride_l, float scale, void* stream, int iters, float* ms_per_launch) {
+    return fa_fwd_timed_ex(q, k, v, mask, out, nullptr, B, R, L, H, stride_b, stride_h, stride_l, stride_b,
+                           stride_h, stride_l, scale, 0, stream, iters, ms_per_launch);
 }
 
 }  // extern "C"

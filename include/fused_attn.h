@@ -141,6 +141,18 @@ int fa_fwd_timed(const void* q, const void* k, const void* v, const void* mask, 
                  float scale, void* stream, int iters, float* ms_per_launch);
 
 /*
+ * fa_fwd_timed for every form of the launch: the arguments of fa_fwd_strided (flags, lse, strides
+ * of `out`) followed by those of the timing loop.  The same counterpart in the reference
+ * (tests/benchmark_fused_attn.py:36-42); fa_fwd_timed is this with lse = NULL, flags = 0 and the
+ * strides of q for out.
+ */
+int fa_fwd_timed_ex(const void* q, const void* k, const void* v, const void* mask, void* out, void* lse,
+                    int64_t B, int64_t R, int64_t L, int64_t H,
+                    int64_t stride_b, int64_t stride_h, int64_t stride_l,
+                    int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_l,
+                    float scale, int flags, void* stream, int iters, float* ms_per_launch);
+
+/*
  * Fused QKV projection, the front end the reference lists as not done (reference README.md:137;
  * its kernel takes queries, keys and values as three separate tensors, reference
  * src/fused_attn_extention.cu:15-22):

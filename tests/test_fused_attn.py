@@ -846,6 +846,79 @@ def test_additive_mask_on_large_grids(gpu, B, R, L, H):
         assert err[keep[b]].max().item() <= TOL, (b, h)
 
 
+def _block_mask(kind, B, L, seed):
+    """Masks under the reference's contract (zero where a pair takes part, -inf where it is muted,
+    reference README.md:88-89), made of large all-zero and all-muted blocks: what the kernels'
+    classification of mask blocks (zero / muted / mixed) is written for."""
+    g = torch.Generator().manual_seed(seed)
+    neg = float("-inf")
+    m = torch.zeros(B, L, L)
+    if kind == "causal":
+        m = torch.full((L, L), neg).triu(1).expand(B, L, L).clone()
+    elif kind == "padding":                     # batch b keeps its first n_b keys
+        for b in range(B):
+            m[b, :, L - 1 - (b * 37 + L // 3) % (L - 1):] = neg
+    elif kind == "documents":                   # block diagonal: three to five documents per batch
+        for b in range(B):
+            cuts = sorted(set(torch.randint(1, L, (4,), generator=g).tolist()) | {0, L})
+            m[b] = neg
+            for lo, hi in zip(cuts[:-1], cuts[1:]):
+                m[b, lo:hi, lo:hi] = 0
+    elif kind in ("blocks", "finite_min"):      # 32 x 32 blocks: 40 % zero, 35 % muted, 25 % element-wise
+        nb = (L + 31) // 32
+        cls = torch.rand(B, nb, nb, generator=g)
+        up = lambda t: t.repeat_interleave(32, 1).repeat_interleave(32, 2)[:, :L, :L]
+        low = -65504.0 if kind == "finite_min" else neg
+        m = torch.where(up(cls) < 0.35, low, 0.0)
+        noisy = torch.where(torch.rand(B, L, L, generator=g) < 0.5, low, 0.0) + torch.randn(B, L, L, generator=g) * 0.25
+        m = torch.where(up(cls) > 0.75, noisy, m)
+        m[:, :, 0] = 0                          # every row keeps a key
+    else:
+        raise ValueError(kind)
+    return m.to(torch.float16)
+
+
+@pytest.mark.parametrize("B,R,L,H", [
+    (4, 16, 2048, 64),       # eight 64-row waves
+    (2, 40, 1024, 128),      # eight 32-row waves, head_dim 128
+    (2, 12, 2048, 64),       # eight 32-row waves, 256-query workgroups
+    (2, 64, 1000, 32),       # ... ragged end
+    (2, 2, 200, 64),         # four waves
+    (1, 4, 1023, 64),        # four waves, element-wise mask loads
+])
+@pytest.mark.parametrize("kind", ["causal", "padding", "documents", "blocks", "finite_min"])
+def test_block_structured_masks(gpu, B, R, L, H, kind):
+    q, k, v = (_rand((B, L, R * H), 5100 + L + i) for i in range(3))
+    mask = _block_mask(kind, B, L, 5110 + L)
+    dead = [(0, min(L - 1, 40)), (B - 1, L - 1)]      # two fully muted rows: zeros, not NaN
+    for b, r in dead:
+        mask[b, r] = float("-inf")
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, mask=mask.to(gpu))
+    assert torch.isfinite(got.float()).all()
+    keep = torch.ones(B, L, dtype=torch.bool)
+    for b, r in dead:
+        assert (got[b, r] == 0).all()
+        mask[b, r] = 0                                # the oracle would give NaN there
+        keep[b, r] = False
+    for b, h in sorted({(0, 0), (B // 2, R // 2), (B - 1, R - 1)}):
+        sl = slice(h * H, (h + 1) * H)
+        want = attention(q[b:b + 1, :, sl], k[b:b + 1, :, sl], v[b:b + 1, :, sl], H, mask=mask[b:b + 1].float())
+        err = (got[b, :, sl].float().cpu() - want[0]).abs()
+        assert err[keep[b]].max().item() <= TOL, (b, h)
+    if kind == "causal":      # the same result as the causal flag, row for row
+        flag = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, causal=True)
+        diff = (flag.float() - got.float()).abs().cpu()
+        assert diff[keep].max().item() <= 2e-3
+
+
+@pytest.mark.parametrize("B,R,L,H", [(4, 16, 2048, 64), (2, 40, 1024, 128), (2, 2, 200, 64)])
+def test_block_structured_masks_bf16(gpu, B, R, L, H):
+    q, k, v = (_rand((B, L, R * H), 5200 + L + i).to(torch.bfloat16) for i in range(3))
+    mask = _block_mask("blocks", B, L, 5210 + L).to(torch.bfloat16)
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, mask=mask.to(gpu))
+    _check_pairs_tol(got, q, k, v, H, [(0, 0), (B - 1, R - 1)], mask.float(), BF16_TOL)
+
+
 # ---- bfloat16 inputs (FA_FLAG_BF16) ------------------------------------------------------------------
 
 BF16_TOL = 2e-2   # bf16 keeps 8 significant bits: the output rounding alone is 2^-9 * |o|
