@@ -12,8 +12,8 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libfused_attn_gfx950.so")
 
 # every symbol include/fused_attn.h declares
-EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_strided", "fa_fwd_plan", "fa_fwd_query", "fa_strerror", "fa_fwd_timed",
-           "fa_fwd_timed_ex", "fa_qkv_proj", "fa_qkv_proj_plan")
+EXPORTS = ("fa_fwd", "fa_fwd_ex", "fa_fwd_strided", "fa_fwd_plan", "fa_fwd_query", "fa_fwd_reference_bias", "fa_strerror",
+           "fa_fwd_timed", "fa_fwd_timed_ex", "fa_qkv_proj", "fa_qkv_proj_plan")
 FLAG_CAUSAL = 1
 FLAG_BF16 = 2
 
@@ -60,6 +60,8 @@ def load_library():
     lib.fa_fwd_plan.restype = ctypes.c_int
     lib.fa_fwd_query.argtypes = [i64]
     lib.fa_fwd_query.restype = ctypes.c_int
+    lib.fa_fwd_reference_bias.argtypes = [i64]
+    lib.fa_fwd_reference_bias.restype = f32
     lib.fa_strerror.argtypes = [ctypes.c_int]
     lib.fa_strerror.restype = ctypes.c_char_p
     _lib = lib

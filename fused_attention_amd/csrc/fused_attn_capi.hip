@@ -309,11 +309,7 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
     p->total_wgs = (int)total;
     p->wgs_per_xcd = (int)((total + fa::kNumXcd - 1) / fa::kNumXcd);
     p->scale_log2e = scale * 1.4426950408889634f;
-    // 11 - ceil(log2 L): a tail of L small weights then loses at most 2^-13 of a row (see kBiasMin)
-    int log2_len = 0;
-    while (((int64_t)1 << log2_len) < L) ++log2_len;
-    const float bias = 11.0f - (float)log2_len;
-    p->bias = bias < fa::kBiasMin ? fa::kBiasMin : (bias > fa::kBiasMax ? fa::kBiasMax : bias);
+    p->bias = fa_fwd_reference_bias(L);
     return FA_OK;
 }
 
@@ -322,6 +318,14 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
 extern "C" {
 
 int fa_fwd_query(int64_t H) { return (H == 16 || H == 32 || H == 64 || H == 128) ? 1 : 0; }
+
+// 11 - ceil(log2 L): a tail of L small weights then loses at most 2^-13 of a row (see kBiasMin)
+float fa_fwd_reference_bias(int64_t L) {
+    int log2_len = 0;
+    while (log2_len < 62 && ((int64_t)1 << log2_len) < L) ++log2_len;
+    const float bias = 11.0f - (float)log2_len;
+    return bias < fa::kBiasMin ? fa::kBiasMin : (bias > fa::kBiasMax ? fa::kBiasMax : bias);
+}
 
 const char* fa_strerror(int status) {
     switch (status) {

@@ -123,6 +123,15 @@ int fa_fwd_plan(int64_t B, int64_t R, int64_t L, int64_t H, int flags, int has_m
 int fa_fwd_query(int64_t H);
 
 /*
+ * The power of two (as a base-2 exponent) the softmax weights of a row of L keys are divided by
+ * before they are rounded to 16 bits for the second product: a key at the running maximum of its
+ * row gets the weight 2^-bias.  11 - ceil(log2 L), kept inside [-8, 6]: see "Accuracy" under fa_fwd.
+ * Exported so that callers and tests can state the accuracy limit of a launch; no counterpart in the
+ * reference, which keeps every intermediate in fp16 (reference include/fused_attn.cuh:174,257,650-653).
+ */
+float fa_fwd_reference_bias(int64_t L);
+
+/*
  * Human-readable text for a status returned by fa_fwd.  Replaces the print-and-exit
  * macros CHECK_CUDA_ERROR / CHECK_LAST_CUDA_ERROR (reference include/fused_attn.cuh:17-42).
  * The returned pointer is static storage.

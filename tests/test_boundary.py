@@ -2,6 +2,7 @@
 declares, rejects bad arguments with status codes before any launch, and the torch binding keeps
 the reference's entry point (reference src/fused_attn_extention.cu:15-22,119-129) and raises on
 arguments the reference rejects (:24-47)."""
+import ctypes
 import inspect
 import os
 import re
@@ -230,16 +231,64 @@ def test_binding_exposes_the_projection_front_end():
         capi.qkv_project(x, w, 1, 64)
     with pytest.raises(ValueError, match="w must have shape"):
         capi.qkv_project(x, w[:, :128], 1, 64)
+    with pytest.raises(ValueError, match="multiple of 64"):
+        capi.qkv_project(x, torch.zeros(64, 96, dtype=torch.float16), 1, 32)      # slices of 32 features
+    with pytest.raises(ValueError, match="F_in"):
+        capi.qkv_project(torch.zeros(1, 64, 96, dtype=torch.float16), torch.zeros(96, 192, dtype=torch.float16), 1, 64)
+    with pytest.raises(ValueError, match="head_dim must be"):
+        capi.qkv_project(x, w, 1, 48)
+    with pytest.raises(ValueError, match="pair"):
+        capi.qkv_project(x, w, 1, 64, rope=torch.zeros(64, 32))                    # one tensor is not a pair of tables
+    # the library's own shape and size codes, through the entry that never launches (pointer and
+    # alignment codes need real allocations: tests/test_qkv_proj.py)
     lib = capi.load_library()
-    ok = 0x1000   # never dereferenced: rejected during validation
-    assert lib.fa_qkv_proj(ok, ok, None, ok, 1, 64, 96, 1, 64, None, None, 0, None) == -3     # F_in not a multiple of 64
-    assert lib.fa_qkv_proj(ok, ok, None, ok, 1, 64, 64, 3, 16, None, None, 0, None) == -3     # R * H not a multiple of 64
-    assert lib.fa_qkv_proj(ok, ok, None, ok, 1, 64, 64, 1, 48, None, None, 0, None) == -2
-    assert lib.fa_qkv_proj(ok, None, None, ok, 1, 64, 64, 1, 64, None, None, 0, None) == -1
-    assert lib.fa_qkv_proj(ok, ok, None, ok, 1, 64, 64, 1, 64, ok, None, 0, None) == -1        # one table without the other
-    assert lib.fa_qkv_proj(ok, ok + 8, None, ok, 1, 64, 64, 1, 64, None, None, 0, None) == -5
-    assert lib.fa_qkv_proj(ok, ok, None, ok, 1, 64, 64, 1, 64, None, None, 1, None) == -7      # causal is not a projection flag
-    assert lib.fa_qkv_proj(ok, ok, None, ok, 2 ** 20, 2 ** 12, 64, 1, 64, None, None, 0, None) == -6
+    out = (ctypes.c_int * 4)()
+    assert lib.fa_qkv_proj_plan(1, 64, 96, 1, 64, out) == -3     # F_in not a multiple of 64
+    assert lib.fa_qkv_proj_plan(1, 64, 64, 3, 16, out) == -3     # R * H not a multiple of 64
+    assert lib.fa_qkv_proj_plan(1, 64, 64, 1, 48, out) == -2
+    assert lib.fa_qkv_proj_plan(1, 0, 64, 1, 64, out) == -3
+    assert lib.fa_qkv_proj_plan(2 ** 20, 2 ** 12, 64, 1, 64, out) == -6
+    assert lib.fa_qkv_proj_plan(1, 64, 64, 1, 64, None) == -1
+    assert lib.fa_qkv_proj_plan(1, 64, 64, 1, 64, out) == 0
+
+
+def test_binding_exposes_the_extensions_of_the_c_abi():
+    """attention_forward_ex: names, defaults, and every rejection that needs no GPU."""
+    import fused_attn
+
+    doc = fused_attn.attention_forward_ex.__doc__
+    names = re.findall(r"(\w+): ", doc.split("->")[0])
+    assert names == ["queries", "keys", "values", "head_dim", "mask", "causal", "return_lse", "layout", "scale"]
+    assert "causal: bool = False" in doc and "return_lse: bool = False" in doc and "layout: str = 'blf'" in doc
+    x = torch.zeros(2, 64, 128, dtype=torch.float16)
+
+    def rejected(match, *args, **kw):
+        with pytest.raises(RuntimeError, match=match):
+            fused_attn.attention_forward_ex(*args, **kw)
+
+    rejected("GPU tensor", x, x, x, 64)
+    rejected("head_dim must be", x, x, x, 48)
+    rejected("float16 or bfloat16", x.float(), x.float(), x.float(), 64)
+    rejected("layout must be", x, x, x, 64, layout="bshd")
+    rejected("takes 4-D", x, x, x, 64, layout="bhld")
+    rejected("takes 3-D", x.view(2, 64, 2, 64), x.view(2, 64, 2, 64), x.view(2, 64, 2, 64), 64)
+    with pytest.raises(TypeError):
+        fused_attn.attention_forward_ex(x, x, 64)
+
+
+def test_reference_bias_follows_the_sequence_length():
+    """11 - ceil(log2 L) inside [-8, 6], as the launcher computes it (exported for this purpose)."""
+    lib = capi.load_library()
+    want = {1: 6, 2: 6, 32: 6, 33: 5, 64: 5, 1000: 1, 1024: 1, 1025: 0, 3073: -1, 4096: -1, 4097: -2, 16384: -3,
+            65536: -5, 65537: -6, 2 ** 19: -8, 2 ** 19 + 1: -8, 2 ** 22: -8, 2 ** 31 - 4097: -8}
+    for L, b in want.items():
+        assert lib.fa_fwd_reference_bias(L) == float(b), L
+    lo = [lib.fa_fwd_reference_bias(L) for L in range(1, 5000)]
+    assert all(a >= b for a, b in zip(lo, lo[1:]))               # never grows with the length
+    # the share of a row that L weights at the bottom of the fp16 range can take: L 2^-(24 - bias)
+    for L in (64, 1000, 4096, 65536, 2 ** 19):
+        assert L * 2.0 ** -(24 - lib.fa_fwd_reference_bias(L)) <= 2.0 ** -13 + 1e-12
+    assert 2 ** 22 * 2.0 ** -(24 + 8) == 2.0 ** -10              # past the clamp the bound loosens: documented
 
 
 def test_binding_rejects_what_the_reference_rejects():

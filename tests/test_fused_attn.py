@@ -789,6 +789,47 @@ def test_heavy_tail_of_small_weights(gpu, B, R, L, H, gap_log2):
     _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R - 1)])
 
 
+@pytest.mark.parametrize("R,L,H", [(8, 65536, 64), (4, 131072, 128)])
+def test_long_sequences_where_the_reference_bias_is_most_negative(gpu, R, L, H):
+    """L = 65536 and 131072: the launcher's bias is -5 and -6 (a key at the reference gets the weight
+    32 or 64), the leash of the speculative reference 10 and 9 log2 units.  Even heads: one dominant
+    key and a heavy tail 17.5 units below it (closed form).  Odd heads: scores that climb by 60
+    log2 units along the key axis, so the reference is rebased again and again (the row then
+    concentrates on the last keys).  Output and log-sum-exp against float32 evaluations of the
+    sampled rows."""
+    B = 1
+    assert capi.load_library().fa_fwd_reference_bias(L) <= -5
+    t = 17.5 / math.log2(math.e) / math.sqrt(H)
+    q = torch.ones(B, L, R * H)
+    k = torch.zeros(B, L, R * H)
+    climb = torch.linspace(0.0, 60.0 / math.log2(math.e) / math.sqrt(H), L)
+    for h in range(R):
+        if h % 2 == 0:
+            k[:, 0, h * H:(h + 1) * H] = t
+        else:
+            k[:, :, h * H:(h + 1) * H] = climb[None, :, None]
+    q, k = q.half(), k.half()
+    v = _rand((B, L, R * H), 6600 + H)
+    v[:, 0] = 4.0
+    got, lse = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, return_lse=True)
+    got, lse = got.float().cpu(), lse.cpu()
+    assert torch.isfinite(got).all() and torch.isfinite(lse).all()
+    rows = torch.tensor([0, 1, 63, 64, 511, 512, L // 2, L - 513, L - 2, L - 1])
+    for h in range(R):
+        sl = slice(h * H, (h + 1) * H)
+        scores = (q[0, rows, sl].float() @ k[0, :, sl].float().T) / math.sqrt(H)
+        want = torch.softmax(scores, dim=-1) @ v[0, :, sl].float()
+        assert (got[0, rows, sl] - want).abs().max().item() <= TOL, h
+        assert (lse[0, h, rows] - torch.logsumexp(scores, dim=-1)).abs().max().item() <= 1e-3 * math.log(L), h
+    # even heads, every row: the closed form
+    gap = k[0, 0, 0].float().item() * math.sqrt(H) * math.log2(math.e)
+    tail = (L - 1) * 2.0 ** -gap
+    for h in range(0, R, 2):
+        sl = slice(h * H, (h + 1) * H)
+        want = (4.0 + tail * v[0, 1:, sl].float().mean(dim=0)) / (1.0 + tail)
+        assert (got[0, :, sl] - want).abs().max().item() <= TOL, h
+
+
 @pytest.mark.parametrize("B,R,L,H", [
     (4, 16, 4096, 64),      # eight-wave workgroups, each taking a pair of query tiles (8 tiles per head)
     (2, 64, 1300, 64),      # ... with an odd number of tiles (the middle one runs alone) and a ragged end
@@ -965,6 +1006,50 @@ def test_bf16_additive_mask_and_closed_forms(gpu, B, R, L, H):
     assert _max_err(zq, want) <= 2e-3
     with pytest.raises(TypeError):
         capi.forward(q.to(gpu), k.half().to(gpu), v.to(gpu), H)
+
+
+@pytest.mark.parametrize("B,R,L,H", [(2, 3, 200, 64), (4, 16, 2048, 64), (2, 40, 1024, 128)])
+def test_extensions_through_the_compiled_module(gpu, B, R, L, H):
+    """fused_attn.attention_forward_ex: causal, mask, log-sum-exp, bf16, the [B, R, L, H] layout and
+    strided views give what capi.forward gives (bit for bit: the same library call) and what the
+    oracle says."""
+    import fused_attn
+
+    q, k, v = (_rand((B, L, R * H), 5300 + L + i) for i in range(3))
+    dq, dk, dv = q.to(gpu), k.to(gpu), v.to(gpu)
+    plain = fused_attn.attention_forward_ex(dq, dk, dv, H)
+    assert isinstance(plain, torch.Tensor) and plain.shape == dq.shape and plain.is_contiguous()
+    assert torch.equal(plain, fused_attn.attention_forward(H, min(128, 2 * H), dq, dk, dv))
+    out, lse = fused_attn.attention_forward_ex(dq, dk, dv, H, causal=True, return_lse=True)
+    want_out, want_lse = capi.forward(dq, dk, dv, H, causal=True, return_lse=True)
+    assert torch.equal(out, want_out) and torch.equal(lse, want_lse) and lse.shape == (B, R, L)
+    _check_pairs(out, q, k, v, H, [(0, 0), (B - 1, R - 1)], mask=causal_mask(B, L))
+    mask = _block_mask("blocks", B, L, 5310 + L)
+    masked = fused_attn.attention_forward_ex(dq, dk, dv, H, mask=mask.to(gpu))
+    assert torch.equal(masked, capi.forward(dq, dk, dv, H, mask=mask.to(gpu)))
+    _check_pairs(masked, q, k, v, H, [(B - 1, R - 1)], mask=mask.float())
+    # [B, R, L, H] views of the same data (no copy), output dense in that layout
+    q4, k4, v4 = (t.view(B, L, R, H).transpose(1, 2) for t in (dq, dk, dv))
+    bhld = fused_attn.attention_forward_ex(q4, k4, v4, H, layout="bhld")
+    assert bhld.shape == (B, R, L, H) and bhld.is_contiguous()
+    assert torch.equal(bhld.transpose(1, 2).reshape(B, L, R * H), plain)
+    # bf16, scale
+    qb, kb, vb = (t.to(torch.bfloat16) for t in (dq, dk, dv))
+    assert torch.equal(fused_attn.attention_forward_ex(qb, kb, vb, H), capi.forward(qb, kb, vb, H))
+    assert torch.equal(fused_attn.attention_forward_ex(dq, dk, dv, H, scale=0.3), capi.forward(dq, dk, dv, H, scale=0.3))
+    # rejections that need device tensors
+    with pytest.raises(RuntimeError, match="cannot be combined"):
+        fused_attn.attention_forward_ex(dq, dk, dv, H, mask=mask.to(gpu), causal=True)
+    with pytest.raises(RuntimeError, match="strides of queries"):
+        fused_attn.attention_forward_ex(dq, torch.zeros(B, L, 2 * R * H, dtype=torch.float16, device=gpu)[:, :, :R * H], dv, H)
+    with pytest.raises(RuntimeError, match="dtype of queries"):
+        fused_attn.attention_forward_ex(dq, kb, dv, H)
+    with pytest.raises(RuntimeError, match="mask must have shape"):
+        fused_attn.attention_forward_ex(dq, dk, dv, H, mask=mask.to(gpu)[:, :, :L - 8].contiguous())
+    with pytest.raises(RuntimeError, match="last dimension"):
+        fused_attn.attention_forward_ex(dq.transpose(1, 2), dk.transpose(1, 2), dv.transpose(1, 2), H)
+    with pytest.raises(RuntimeError, match="scale must be"):
+        fused_attn.attention_forward_ex(dq, dk, dv, H, scale=-1.0)
 
 
 def test_causal_with_mask_is_rejected(gpu):

@@ -153,6 +153,31 @@ def test_projection_through_the_torch_binding(gpu):
         fused_attn.qkv_projection(x.to(gpu), w[:, :64].contiguous().to(gpu), None, R, H)
     with pytest.raises(RuntimeError, match="GPU tensor"):
         fused_attn.qkv_projection(x, w, None, R, H)
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        fused_attn.qkv_projection(x.to(gpu), w[:, :96].contiguous().to(gpu), None, 1, 32)
+
+
+@pytest.mark.parametrize("B,L,Fin,R,H,causal", [(2, 200, 128, 2, 64, False), (2, 1024, 512, 8, 64, True),
+                                                 (1, 2048, 256, 16, 128, False)])
+def test_projection_into_attention_through_the_compiled_module(gpu, B, L, Fin, R, H, causal):
+    """fused_attn.qkv_projection -> fused_attn.attention_forward_ex on the three slices of the packed
+    tensor, no copy in between, against oracle projection + oracle attention."""
+    import fused_attn
+    from oracle import attention, causal_mask
+
+    x, w, b = _rand((B, L, Fin), 7600), _rand((Fin, 3 * R * H), 7601, 1.0 / math.sqrt(Fin)), _rand((3 * R * H,), 7602, 0.1)
+    cos, sin = rope_tables(L, H)
+    qkv = fused_attn.qkv_projection(x.to(gpu), w.to(gpu), b.to(gpu), R, H, cos.to(gpu), sin.to(gpu))
+    views = [qkv[:, :, s] for s in range(3)]
+    assert all(not t.is_contiguous() and t.data_ptr() == qkv.data_ptr() + s * R * H * 2 for s, t in enumerate(views))
+    out = fused_attn.attention_forward_ex(*views, H, causal=causal)
+    assert out.shape == (B, L, R * H) and out.is_contiguous()
+    ref = qkv_projection(x, w, b, R, H, cos, sin)                 # float32 [B, L, 3, R H]
+    ref = ref.to(torch.float16).float()                           # the kernel's q, k, v are rounded to fp16
+    want = attention(ref[:, :, 0].contiguous(), ref[:, :, 1].contiguous(), ref[:, :, 2].contiguous(), H,
+                     mask=causal_mask(B, L) if causal else None)
+    assert torch.isfinite(out.float()).all()
+    assert (out.float().cpu() - want).abs().max().item() <= 5e-3
 
 
 def test_projection_and_attention_captured_in_one_graph(gpu):
