@@ -15,7 +15,7 @@ time, TFLOP/s, roofline fraction and error on a bounded sample for the other con
 the QKV projection front end.
 
 usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5a|c5b|readme] [--causal]
-                       [--others auto|on|off]
+                       [--mask causal|zero] [--projection plain|rotary] [--others auto|on|off]
 """
 import argparse
 import json
@@ -36,6 +36,7 @@ PEAK_TFLOPS_FP16 = 2500.0   # MI355X dense fp16 MFMA, published
 # counter run report null.
 MEASURED_TRAFFIC = {
     "c3": (134.4e6, "profiles/fwd_kernel_pingpong_c3.md"),
+    "c3_mask": (921.2e6, "profiles/fwd_kernel_pingpong_mask.md"),
     "c4": (806.5e6, "profiles/fwd_kernel_pingpong_c4.md"),
     "readme": (335.7e6, "profiles/fwd_kernel_pingpong_readme.md"),
     "qkv_proj_c3": (269.4e6, "profiles/qkv_proj_kernel_c3.md"),
@@ -290,6 +291,10 @@ def main():
     ap.add_argument("--causal", action="store_true",
                     help="the causal extension of the C ABI instead of the reference's non-causal forward: "
                          "counts the flops of the keys at or below the diagonal, no CPU baseline")
+    ap.add_argument("--mask", choices=["causal", "zero"], default=None,
+                    help="the additive-mask path instead of the plain forward: an fp16 [B, L, L] mask of zeros below "
+                         "and -inf above the diagonal (the causal result; counts the flops of the pairs at or below "
+                         "the diagonal), or a mask of zeros (the plain result, all flops); no CPU baseline")
     ap.add_argument("--calibration-copy-mib", type=int, default=1024,
                     help="size of the plain copy run before the timed region (0 disables it)")
     ap.add_argument("--cpu-budget-s", type=float, default=15.0,
@@ -342,11 +347,18 @@ def main():
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     chunk = min(128, w.H * 2)
 
-    if args.causal:
+    if args.causal and args.mask:
+        sys.exit("--causal and --mask are two ways to the same result: pick one")
+    mask = None
+    if args.mask == "causal":
+        mask = torch.full((w.L, w.L), float("-inf")).triu(1).to(torch.float16).expand(w.B, w.L, w.L).contiguous().to(dev)
+    elif args.mask == "zero":
+        mask = torch.zeros(w.B, w.L, w.L, dtype=torch.float16, device=dev)
+    if args.causal or mask is not None:
         out = torch.empty_like(qd)
 
         def step():
-            return capi.forward(qd, kd, vd, w.H, out=out, causal=True)
+            return capi.forward(qd, kd, vd, w.H, out=out, causal=args.causal, mask=mask)
     else:
         def step():
             return fused_attn.attention_forward(w.H, chunk, qd, kd, vd)
@@ -368,14 +380,17 @@ def main():
     out, ms_per_step = timed_steps()
 
     # Kernel duration: HIP events on the launch stream around back-to-back launches, inside the library.
-    kernel_ms = capi.forward_timed(qd, kd, vd, w.H, out, iters=args.steps, causal=args.causal)
+    kernel_ms = capi.forward_timed(qd, kd, vd, w.H, out, iters=args.steps, causal=args.causal, mask=mask)
 
-    # causal: query i attends to i + 1 keys
-    flop = 2.0 * w.B * w.R * w.L * (w.L + 1) * w.H if args.causal else workloads.flops(w)
+    # causal (flag or mask pattern): query i attends to i + 1 keys
+    half = args.causal or args.mask == "causal"
+    variant = "causal" if args.causal else ("additive mask (%s pattern)" % args.mask if args.mask else "non-causal")
+    flop = 2.0 * w.B * w.R * w.L * (w.L + 1) * w.H if half else workloads.flops(w)
     value = flop / (ms_per_step * 1e-3) / 1e12
     achieved = flop / (kernel_ms * 1e-3) / 1e12
+    traffic_key = w.name + ("_causal" if args.causal else "_mask" if args.mask == "causal" else "_mask_zero" if args.mask else "")
     line = {
-        "metric": "fused attn fwd causal TFLOP/s (2*B*R*L*(L+1)*H)" if args.causal else "fused attn fwd TFLOP/s (4*B*R*L^2*H)",
+        "metric": "fused attn fwd causal TFLOP/s (2*B*R*L*(L+1)*H)" if half else "fused attn fwd TFLOP/s (4*B*R*L^2*H)",
         "value": value,
         "unit": "TFLOP/s",
         "pct_of_fp16_mfma_peak": 100.0 * value / PEAK_TFLOPS_FP16,
@@ -393,8 +408,7 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "%s: B=%d R=%d L=%d H=%d %s, fp16 N(0,%g) seeded on the host, "
-                        "fed as [B, L, R*H]" % (w.name, w.B, w.R, w.L, w.H, "causal" if args.causal else "non-causal",
-                                                w.q_std),
+                        "fed as [B, L, R*H]" % (w.name, w.B, w.R, w.L, w.H, variant, w.q_std),
             "flop_per_step": flop,
             "bytes_per_step": workloads.io_bytes(w),
         },
@@ -404,14 +418,14 @@ def main():
             "peak": PEAK_TFLOPS_FP16,
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_TFLOPS_FP16,
-            "traffic": None if args.causal else MEASURED_TRAFFIC.get(w.name, (None, None))[0],
-            "traffic_source": None if args.causal else MEASURED_TRAFFIC.get(w.name, (None, None))[1],
+            "traffic": MEASURED_TRAFFIC.get(traffic_key, (None, None))[0],
+            "traffic_source": MEASURED_TRAFFIC.get(traffic_key, (None, None))[1],
             "kernel_ms": kernel_ms,
         },
     }
-    if args.cpu_budget_s > 0 and not args.causal:
+    if args.cpu_budget_s > 0 and not args.causal and mask is None:
         line["cpu_baseline"] = cpu_baseline(w, q, k, v, out, args.cpu_budget_s)
-    others = args.others == "on" or (args.others == "auto" and args.workload == "c3" and not args.causal)
+    others = args.others == "on" or (args.others == "auto" and args.workload == "c3" and not args.causal and mask is None)
     if others:
         del qd, kd, vd, out
         torch.cuda.empty_cache()
