@@ -79,9 +79,9 @@ def _check(status):
 
 def launch_plan(B, R, L, H, causal=False, has_mask=False):
     """What fa_fwd_plan reports for a problem, as a dict.  Needs no GPU."""
-    out = (ctypes.c_int * 6)()
+    out = (ctypes.c_int * 7)()
     _check(load_library().fa_fwd_plan(B, R, L, H, FLAG_CAUSAL if causal else 0, 1 if has_mask else 0, out))
-    keys = ("waves", "rows_per_wave", "workgroups", "working", "per_head", "heads_per_xcd")
+    keys = ("waves", "rows_per_wave", "workgroups", "working", "per_head", "heads_per_xcd", "matrix_tile")
     return dict(zip(keys, out))
 
 

@@ -199,6 +199,30 @@ hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
     return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(NW * 64), args, lds, stream);
 }
 
+// The eight-wave kernel with its products written as 16 x 16 tiles (fwd_kernel_pp16): plain launches
+// at head_dim 64 made of whole rounds of workgroups.  On a full chip the clock follows the switching
+// activity and the 16 x 16 x 32 instruction moves half as many accumulator registers per flop
+// (measured, same box: 256 workgroups +2.9 and +3.6 %, 512 +3.5 %, 480 +1.1 %); where part of the
+// chip idles the clock is not held back and its 36 matrix instructions per sub-tile instead of 20
+// cost more than they save, and a part-filled last round takes that from the whole launch (192
+// workgroups -5 to -9 %, 384 -3.4 and -4.6 %, 448 -0.7 %, 640 -1.0 %, 1152 -0.8 %).  Taken when the
+// last round is at least seven eighths full.
+bool use_tiles16(int64_t H, Shape sh, const fa::FwdParams& p) {
+    if (H != 64 || sh.waves != 8 || sh.nqb != 2) return false;
+    const int last = p.total_wgs % kNumCu;
+    return p.total_wgs >= kNumCu && (last == 0 || 8 * last >= 7 * kNumCu);
+}
+
+template <bool BF>
+hipError_t launch_pp16(const fa::FwdParams& p, hipStream_t stream) {
+    constexpr int lds = fa::lds_bytes_pingpong<64, 2>();
+    auto kernel = BF ? fa::bf16::fwd_kernel_pp16<8, true> : fa::fwd_kernel_pp16<8, true>;
+    fa::FwdParams params = p;
+    void* args[] = {&params};
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(p.wgs_per_xcd * fa::kNumXcd), dim3(8 * 64), args,
+                           lds, stream);
+}
+
 template <int H, int MODE, bool BF>
 hipError_t dispatch_shape(Shape sh, const fa::FwdParams& p, hipStream_t stream) {
     // the dealt causal schedule exists for the eight-wave kernel at head_dim 64 and 128 only
@@ -366,6 +390,8 @@ int fa_fwd_strided(const void* q, const void* k, const void* v, const void* mask
         e = p.heads_per_xcd > 0 ? dispatch<fa::kCausalDealt>(H, shape, p, s, bf16) : dispatch<fa::kCausal>(H, shape, p, s, bf16);
     else if (mask != nullptr)
         e = dispatch<fa::kAdditive>(H, shape, p, s, bf16);
+    else if (use_tiles16(H, shape, p))
+        e = bf16 ? launch_pp16<true>(p, s) : launch_pp16<false>(p, s);
     else
         e = dispatch<fa::kPlain>(H, shape, p, s, bf16);
     return static_cast<int>(e);
@@ -390,6 +416,7 @@ int fa_fwd_plan(int64_t B, int64_t R, int64_t L, int64_t H, int flags, int has_m
     plan[3] = p.total_wgs;
     plan[4] = p.n_qtiles;
     plan[5] = p.heads_per_xcd;
+    plan[6] = (!causal && !has_mask && use_tiles16(H, shape, p)) ? 16 : 32;
     return FA_OK;
 }
 

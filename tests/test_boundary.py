@@ -198,6 +198,22 @@ def test_benchmark_workloads_take_the_kernels_the_documentation_names():
     assert plan(64, 12, 128, 64, has_mask=True) == (4, 32, False)
 
 
+def test_the_16_row_matrix_tile_is_taken_on_whole_rounds_only():
+    tile = lambda B, R, L, H, **kw: capi.launch_plan(B, R, L, H, **kw)["matrix_tile"]
+    wgs = lambda B, R, L, H: capi.launch_plan(B, R, L, H)["working"]
+    assert (wgs(4, 16, 4096, 64), tile(4, 16, 4096, 64)) == (512, 16)     # c3: two whole rounds
+    assert (wgs(4, 16, 2048, 64), tile(4, 16, 2048, 64)) == (256, 16)     # one whole round
+    assert (wgs(8, 32, 1000, 64), tile(8, 32, 1000, 64)) == (512, 16)     # ragged tiles make no difference
+    assert (wgs(2, 60, 2048, 64), tile(2, 60, 2048, 64)) == (480, 16)     # last round seven eighths full
+    assert (wgs(2, 56, 2048, 64), tile(2, 56, 2048, 64)) == (448, 32)     # ... three quarters full
+    assert (wgs(6, 16, 2048, 64), tile(6, 16, 2048, 64)) == (384, 32)     # one and a half rounds
+    assert (wgs(9, 16, 4096, 64), tile(9, 16, 4096, 64)) == (1152, 32)    # four and a half
+    assert (wgs(8, 12, 1024, 64), tile(8, 12, 1024, 64)) == (192, 32)     # c2: less than one round
+    assert tile(4, 16, 4096, 64, causal=True) == 32                       # plain launches only
+    assert tile(4, 16, 4096, 64, has_mask=True) == 32
+    assert tile(4, 32, 4096, 32) == 32 and tile(1, 32, 16384, 128) == 32  # head_dim 64 only
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(capi, "_lib", None)
     monkeypatch.setattr(capi, "LIB_PATH", os.path.join(REPO, "does_not_exist.so"))

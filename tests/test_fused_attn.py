@@ -718,6 +718,35 @@ def test_launch_shapes_plain(gpu, B, R, L, H):
     _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R // 2), (B - 1, R - 1)])
 
 
+@pytest.mark.parametrize("B,R,L", [
+    (4, 16, 2048),      # one whole round of 512-query workgroups
+    (8, 32, 1000),      # two rounds, ragged last key tile and second query tile
+    (4, 64, 1500),      # three rounds, three tiles per head, the last a quarter full
+    (2, 60, 2048),      # a last round seven eighths full
+    (1, 16, 16384),     # long rows: 256 key tiles per workgroup
+])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_kernel_with_16_row_matrix_tiles(gpu, B, R, L, dtype):
+    # Plain launches at head_dim 64 whose workgroups fill whole rounds of the chip take the kernel
+    # written on 16 x 16 x 32 products; here with row log-sum-exps, in both layouts.
+    H = 64
+    assert capi.launch_plan(B, R, L, H)["matrix_tile"] == 16
+    q, k, v = (_rand((B, L, R * H), 4000 + L + i).to(dtype) for i in range(3))
+    got, lse = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, return_lse=True)
+    assert torch.isfinite(got.float()).all()
+    tol = TOL if dtype == torch.float16 else BF16_TOL
+    pairs = [(0, 0), (B // 2, R // 3), (B - 1, R // 2), (B - 1, R - 1)]
+    for b, h in pairs:
+        sl = slice(h * H, (h + 1) * H)
+        want = attention(q[b:b + 1, :, sl], k[b:b + 1, :, sl], v[b:b + 1, :, sl], H)
+        assert _max_err(got[b:b + 1, :, sl], want) <= tol, (b, h)
+        want = attention_lse(q[b:b + 1, :, sl], k[b:b + 1, :, sl], H)[0, 0]
+        assert ((lse[b, h].cpu() - want).abs() / (1 + want.abs())).max().item() <= 1e-3, (b, h)
+    heads = lambda t: t.view(B, L, R, H).permute(0, 2, 1, 3).contiguous().to(gpu)
+    same = capi.forward(heads(q), heads(k), heads(v), H, layout="bhld")
+    assert torch.equal(same.permute(0, 2, 1, 3).reshape(B, L, R * H), got)
+
+
 @pytest.mark.parametrize("B,R,L,H", [(4, 16, 2048, 64), (2, 64, 1024, 128)])
 @pytest.mark.parametrize("kind", ["std3", "rising", "falling"])
 def test_eight_wave_kernel_on_adversarial_scores(gpu, B, R, L, H, kind):
