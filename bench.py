@@ -35,7 +35,7 @@ PEAK_TFLOPS_FP16 = 2500.0   # MI355X dense fp16 MFMA, published
 # write) and are quoted here with the file that holds the counter summary.  Workloads without a
 # counter run report null.
 MEASURED_TRAFFIC = {
-    "c3": (134.4e6, "profiles/fwd_kernel_pingpong_c3.md"),
+    "c3": (134.4e6, "profiles/fwd_kernel_pp16_c3.md"),
     "c3_mask": (921.2e6, "profiles/fwd_kernel_pingpong_mask.md"),
     "c4": (806.5e6, "profiles/fwd_kernel_pingpong_c4.md"),
     "readme": (335.7e6, "profiles/fwd_kernel_pingpong_readme.md"),
