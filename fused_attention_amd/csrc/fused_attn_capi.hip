@@ -213,10 +213,11 @@ bool use_tiles16(int64_t H, Shape sh, const fa::FwdParams& p) {
     return p.total_wgs >= kNumCu && (last == 0 || 8 * last >= 7 * kNumCu);
 }
 
-template <bool BF>
+template <bool BF, bool CAUSAL>
 hipError_t launch_pp16(const fa::FwdParams& p, hipStream_t stream) {
     constexpr int lds = fa::lds_bytes_pingpong<64, 2>();
-    auto kernel = BF ? fa::bf16::fwd_kernel_pp16<8, true> : fa::fwd_kernel_pp16<8, true>;
+    // (the causal form has one score buffer: its loops take the parity of a sub-tile at run time)
+    auto kernel = BF ? fa::bf16::fwd_kernel_pp16<8, !CAUSAL, CAUSAL> : fa::fwd_kernel_pp16<8, !CAUSAL, CAUSAL>;
     fa::FwdParams params = p;
     void* args[] = {&params};
     return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(p.wgs_per_xcd * fa::kNumXcd), dim3(8 * 64), args,
@@ -386,12 +387,16 @@ int fa_fwd_strided(const void* q, const void* k, const void* v, const void* mask
     if (rc != FA_OK) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e;
-    if (causal)
-        e = p.heads_per_xcd > 0 ? dispatch<fa::kCausalDealt>(H, shape, p, s, bf16) : dispatch<fa::kCausal>(H, shape, p, s, bf16);
+    if (causal && p.heads_per_xcd > 0)
+        e = dispatch<fa::kCausalDealt>(H, shape, p, s, bf16);
+    else if (causal && use_tiles16(H, shape, p))     // whole rounds of pairs of query tiles
+        e = bf16 ? launch_pp16<true, true>(p, s) : launch_pp16<false, true>(p, s);
+    else if (causal)
+        e = dispatch<fa::kCausal>(H, shape, p, s, bf16);
     else if (mask != nullptr)
         e = dispatch<fa::kAdditive>(H, shape, p, s, bf16);
     else if (use_tiles16(H, shape, p))
-        e = bf16 ? launch_pp16<true>(p, s) : launch_pp16<false>(p, s);
+        e = bf16 ? launch_pp16<true, false>(p, s) : launch_pp16<false, false>(p, s);
     else
         e = dispatch<fa::kPlain>(H, shape, p, s, bf16);
     return static_cast<int>(e);
@@ -416,7 +421,7 @@ int fa_fwd_plan(int64_t B, int64_t R, int64_t L, int64_t H, int flags, int has_m
     plan[3] = p.total_wgs;
     plan[4] = p.n_qtiles;
     plan[5] = p.heads_per_xcd;
-    plan[6] = (!causal && !has_mask && use_tiles16(H, shape, p)) ? 16 : 32;
+    plan[6] = (!has_mask && p.heads_per_xcd == 0 && use_tiles16(H, shape, p)) ? 16 : 32;
     return FA_OK;
 }
 

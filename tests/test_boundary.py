@@ -209,8 +209,11 @@ def test_the_16_row_matrix_tile_is_taken_on_whole_rounds_only():
     assert (wgs(6, 16, 2048, 64), tile(6, 16, 2048, 64)) == (384, 32)     # one and a half rounds
     assert (wgs(9, 16, 4096, 64), tile(9, 16, 4096, 64)) == (1152, 32)    # four and a half
     assert (wgs(8, 12, 1024, 64), tile(8, 12, 1024, 64)) == (192, 32)     # c2: less than one round
-    assert tile(4, 16, 4096, 64, causal=True) == 32                       # plain launches only
-    assert tile(4, 16, 4096, 64, has_mask=True) == 32
+    assert tile(4, 16, 4096, 64, causal=True) == 16                       # causal: whole rounds of pairs of tiles
+    assert tile(2, 85, 2500, 64, causal=True) == 16                       # ... 510 pairs and lone middle tiles
+    assert tile(2, 64, 1300, 64, causal=True) == 32                       # ... but not where the tiles are dealt out
+    assert tile(4, 16, 2048, 64, causal=True) == 32                       # 128 pairs: half a round
+    assert tile(4, 16, 4096, 64, has_mask=True) == 32                     # never with a mask
     assert tile(4, 32, 4096, 32) == 32 and tile(1, 32, 16384, 128) == 32  # head_dim 64 only
 
 

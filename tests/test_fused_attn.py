@@ -747,6 +747,37 @@ def test_kernel_with_16_row_matrix_tiles(gpu, B, R, L, dtype):
     assert torch.equal(same.permute(0, 2, 1, 3).reshape(B, L, R * H), got)
 
 
+@pytest.mark.parametrize("B,R,L", [
+    (4, 16, 4096),      # 256 pairs of 512-query tiles
+    (16, 16, 1024),     # one pair per head: both tiles are diagonal tiles
+    (16, 16, 1000),     # ... with a ragged second tile
+    (2, 85, 2500),      # five tiles per head: two pairs and the middle tile alone, ragged end
+    (1, 16, 16384),     # 16 pairs per head, up to 32 key tiles below the diagonal
+])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_causal_kernel_with_16_row_matrix_tiles(gpu, B, R, L, dtype):
+    # Causal launches at head_dim 64 made of whole rounds of pairs of query tiles: the 16 x 16 kernel,
+    # whose waves own blocks of 16 queries dealt out so that all eight reach their diagonals together.
+    H = 64
+    assert capi.launch_plan(B, R, L, H, causal=True)["matrix_tile"] == 16
+    q, k, v = (_rand((B, L, R * H), 4050 + L + i).to(dtype) for i in range(3))
+    got, lse = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, causal=True, return_lse=True)
+    assert torch.isfinite(got.float()).all()
+    assert torch.equal(got[:, 0].cpu(), v[:, 0])           # the first query sees the first key only
+    tol = TOL if dtype == torch.float16 else BF16_TOL
+    mask = causal_mask(1, L)
+    for b, h in [(0, 0), (B // 2, R // 3), (B - 1, R - 1)]:
+        sl = slice(h * H, (h + 1) * H)
+        want = attention(q[b:b + 1, :, sl], k[b:b + 1, :, sl], v[b:b + 1, :, sl], H, mask=mask)
+        assert _max_err(got[b:b + 1, :, sl], want) <= tol, (b, h)
+        want = attention_lse(q[b:b + 1, :, sl], k[b:b + 1, :, sl], H, mask=mask)[0, 0]
+        assert ((lse[b, h].cpu() - want).abs() / (1 + want.abs())).max().item() <= 1e-3, (b, h)
+    # the same rows through the additive-mask path (the 32 x 32 kernel): two kernels, one result
+    if L <= 4096:
+        other = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, mask=causal_mask(B, L).to(dtype).to(gpu))
+        assert (other.float() - got.float()).abs().max().item() <= (2e-3 if dtype == torch.float16 else BF16_TOL)
+
+
 @pytest.mark.parametrize("B,R,L,H", [(4, 16, 2048, 64), (2, 64, 1024, 128)])
 @pytest.mark.parametrize("kind", ["std3", "rising", "falling"])
 def test_eight_wave_kernel_on_adversarial_scores(gpu, B, R, L, H, kind):
