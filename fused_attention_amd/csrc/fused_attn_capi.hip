@@ -216,8 +216,7 @@ bool use_tiles16(int64_t H, Shape sh, const fa::FwdParams& p) {
 template <bool BF, bool CAUSAL>
 hipError_t launch_pp16(const fa::FwdParams& p, hipStream_t stream) {
     constexpr int lds = fa::lds_bytes_pingpong<64, 2>();
-    // (the causal form has one score buffer: its loops take the parity of a sub-tile at run time)
-    auto kernel = BF ? fa::bf16::fwd_kernel_pp16<8, !CAUSAL, CAUSAL> : fa::fwd_kernel_pp16<8, !CAUSAL, CAUSAL>;
+    auto kernel = BF ? fa::bf16::fwd_kernel_pp16<8, true, CAUSAL> : fa::fwd_kernel_pp16<8, true, CAUSAL>;
     fa::FwdParams params = p;
     void* args[] = {&params};
     return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(p.wgs_per_xcd * fa::kNumXcd), dim3(8 * 64), args,
