@@ -310,6 +310,12 @@ int validate(const void* q, const void* k, const void* v, const void* mask, void
             total = kNumCu;                                           // a resident grid
         }
     }
+    if (mask != nullptr && shape->waves == 8 && n_qtiles > 1) {
+        // Pairs of query tiles for a masked launch of the eight-wave kernel (see the kernel) when the
+        // pairs, two tiles long, need no more time on the chip than the tiles in rounds of their own
+        const int64_t pairs = (n_qtiles + 1) / 2;
+        if (2 * ceil_div(B * R * pairs, kNumCu) <= ceil_div(B * R * n_qtiles, kNumCu)) n_qtiles = pairs;
+    }
     if (total == 0) total = B * R * n_qtiles;
     if (total > kMaxInt - 8 || B * R > kMaxInt) return FA_ERR_TOO_LARGE;
     if (!extent_ok(in, B, R, L) || !extent_ok(os, B, R, L)) return FA_ERR_TOO_LARGE;

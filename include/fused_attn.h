@@ -109,7 +109,8 @@ int fa_fwd_strided(const void* q, const void* k, const void* v, const void* mask
  * tests of the launcher and for tuning.  has_mask != 0 stands for an additive mask with 16-byte
  * aligned rows.  Fills plan[0..6] with: wave64s per workgroup; query rows per wave; workgroups
  * launched; workgroups that do work (the rest exit at once); workgroups per (batch, head), or
- * pairs of query tiles per head for a causal launch of the eight-wave kernel; 0, or, when the
+ * pairs of query tiles per head for a causal launch of the eight-wave kernel and for those masked
+ * launches of it that pairs cost no round of the chip; 0, or, when the
  * query tiles of a causal launch are dealt out to a resident grid, the heads per XCD; the edge of
  * the matrix instruction's tile, 32, or 16 for plain launches at head_dim 64 whose workgroups fill
  * whole rounds of the chip (the last round at least seven eighths full).

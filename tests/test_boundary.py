@@ -92,7 +92,7 @@ def _items_of_plan(plan, heads, L, causal):
                     break
                 items.append((wg % 8 + 8 * (j % plan["heads_per_xcd"]), tiles - 1 - j // plan["heads_per_xcd"]))
                 rnd += 1
-        elif causal and plan["waves"] == 8:                # causal, a pair of tiles per workgroup
+        elif plan["waves"] == 8 and (causal or plan["per_head"] < tiles):   # a pair of tiles per workgroup (causal; some masked launches)
             head, slot = divmod(logical, plan["per_head"])
             items.append((head, tiles - 1 - slot))
             if 2 * slot != tiles - 1:
@@ -120,7 +120,7 @@ def test_every_launch_plan_covers_every_query_tile_once():
         heads = rng.choice([1, 3, 8, 12, 16, 20, 24, 40, 48, 64, 80, 96, 120, 160, 256, 320, 640])
         B = rng.choice([b for b in (1, 2, 4, 8) if heads % b == 0])
         shapes.append((B, heads // B, L, H))
-    dealt = 0
+    dealt = paired_masks = 0
     for B, R, L, H in shapes:
         for causal, has_mask in ((False, False), (True, False), (False, True)):
             if has_mask and L % 8:
@@ -132,7 +132,11 @@ def test_every_launch_plan_covers_every_query_tile_once():
             assert len(items) == B * R * tiles, (B, R, L, H, causal, has_mask, plan)
             assert set(items) == {(h, t) for h in range(B * R) for t in range(tiles)}, (B, R, L, H, causal, has_mask, plan)
             dealt += plan["heads_per_xcd"] > 0
+            paired_masks += has_mask and plan["waves"] == 8 and plan["per_head"] < tiles
+            if not causal and not has_mask:
+                assert plan["per_head"] == tiles
     assert dealt > 10          # the dealt schedule was among the plans
+    assert paired_masks > 10   # ... and masked launches in pairs of tiles
 
 
 def _tiles_of_projection_plan(plan):
