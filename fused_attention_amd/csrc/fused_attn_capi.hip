@@ -199,24 +199,28 @@ hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
     return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(NW * 64), args, lds, stream);
 }
 
-// The eight-wave kernel with its products written as 16 x 16 tiles (fwd_kernel_pp16): plain launches
-// at head_dim 64 made of whole rounds of workgroups.  On a full chip the clock follows the switching
-// activity and the 16 x 16 x 32 instruction moves half as many accumulator registers per flop
-// (measured, same box: 256 workgroups +2.9 and +3.6 %, 512 +3.5 %, 480 +1.1 %); where part of the
-// chip idles the clock is not held back and its 36 matrix instructions per sub-tile instead of 20
-// cost more than they save, and a part-filled last round takes that from the whole launch (192
-// workgroups -5 to -9 %, 384 -3.4 and -4.6 %, 448 -0.7 %, 640 -1.0 %, 1152 -0.8 %).  Taken when the
-// last round is at least seven eighths full.
-bool use_tiles16(int64_t H, Shape sh, const fa::FwdParams& p) {
+// The eight-wave kernel with its products written as 16 x 16 tiles (fwd_kernel_pp16), head_dim 64.
+// Plain launches: on a full chip the clock follows the switching activity and the 16 x 16 x 32
+// instruction moves half as many accumulator registers per flop (measured, same box: 256
+// workgroups +2.9 and +3.6 %, 512 +3.5 %, 480 +1.1 %); where part of the chip idles the clock is not
+// held back and its 36 matrix instructions per sub-tile instead of 20 cost more than they save, and
+// a part-filled last round takes that from the whole launch (192 workgroups -5 to -9 %, 384 -3.4
+// and -4.6 %, 448 -0.7 %, 640 -1.0 %, 1152 -0.8 %): taken when the last round is at least seven
+// eighths full.  Causal launches in pairs of tiles: there the gain is the kernel's deal of 16-query
+// blocks to the waves, which does not depend on the clock, and only an emptier single round loses
+// (144 pairs -4.3 %, 160 -6.2 %, 192 -1.4 and +1.3 %, 200 -0.6 %; 240 +3.6 %, 256 +5.5 %, 400
+// +1.4 %, 960 +4.5 and +7.5 %, 1152 +5.4 %): taken from seven eighths of a round on.
+bool use_tiles16(int64_t H, Shape sh, const fa::FwdParams& p, bool causal) {
     if (H != 64 || sh.waves != 8 || sh.nqb != 2) return false;
+    if (causal) return 8 * (int64_t)p.total_wgs >= 7 * kNumCu;     // (a dealt launch is a whole resident grid)
     const int last = p.total_wgs % kNumCu;
     return p.total_wgs >= kNumCu && (last == 0 || 8 * last >= 7 * kNumCu);
 }
 
-template <bool BF, bool CAUSAL>
+template <bool BF, int MODE>
 hipError_t launch_pp16(const fa::FwdParams& p, hipStream_t stream) {
     constexpr int lds = fa::lds_bytes_pingpong<64, 2>();
-    auto kernel = BF ? fa::bf16::fwd_kernel_pp16<8, true, CAUSAL> : fa::fwd_kernel_pp16<8, true, CAUSAL>;
+    auto kernel = BF ? fa::bf16::fwd_kernel_pp16<8, true, MODE> : fa::fwd_kernel_pp16<8, true, MODE>;
     fa::FwdParams params = p;
     void* args[] = {&params};
     return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(p.wgs_per_xcd * fa::kNumXcd), dim3(8 * 64), args,
@@ -392,16 +396,18 @@ int fa_fwd_strided(const void* q, const void* k, const void* v, const void* mask
     if (rc != FA_OK) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e;
-    if (causal && p.heads_per_xcd > 0)
+    if (causal && use_tiles16(H, shape, p, true) && p.heads_per_xcd > 0)
+        e = bf16 ? launch_pp16<true, fa::kCausalDealt>(p, s) : launch_pp16<false, fa::kCausalDealt>(p, s);
+    else if (causal && use_tiles16(H, shape, p, true))
+        e = bf16 ? launch_pp16<true, fa::kCausal>(p, s) : launch_pp16<false, fa::kCausal>(p, s);
+    else if (causal && p.heads_per_xcd > 0)
         e = dispatch<fa::kCausalDealt>(H, shape, p, s, bf16);
-    else if (causal && use_tiles16(H, shape, p))     // whole rounds of pairs of query tiles
-        e = bf16 ? launch_pp16<true, true>(p, s) : launch_pp16<false, true>(p, s);
     else if (causal)
         e = dispatch<fa::kCausal>(H, shape, p, s, bf16);
     else if (mask != nullptr)
         e = dispatch<fa::kAdditive>(H, shape, p, s, bf16);
-    else if (use_tiles16(H, shape, p))
-        e = bf16 ? launch_pp16<true, false>(p, s) : launch_pp16<false, false>(p, s);
+    else if (use_tiles16(H, shape, p, false))
+        e = bf16 ? launch_pp16<true, fa::kPlain>(p, s) : launch_pp16<false, fa::kPlain>(p, s);
     else
         e = dispatch<fa::kPlain>(H, shape, p, s, bf16);
     return static_cast<int>(e);
@@ -426,7 +432,7 @@ int fa_fwd_plan(int64_t B, int64_t R, int64_t L, int64_t H, int flags, int has_m
     plan[3] = p.total_wgs;
     plan[4] = p.n_qtiles;
     plan[5] = p.heads_per_xcd;
-    plan[6] = (!has_mask && p.heads_per_xcd == 0 && use_tiles16(H, shape, p)) ? 16 : 32;
+    plan[6] = (!has_mask && use_tiles16(H, shape, p, causal)) ? 16 : 32;
     return FA_OK;
 }
 

@@ -215,8 +215,11 @@ def test_the_16_row_matrix_tile_is_taken_on_whole_rounds_only():
     assert (wgs(8, 12, 1024, 64), tile(8, 12, 1024, 64)) == (192, 32)     # c2: less than one round
     assert tile(4, 16, 4096, 64, causal=True) == 16                       # causal: whole rounds of pairs of tiles
     assert tile(2, 85, 2500, 64, causal=True) == 16                       # ... 510 pairs and lone middle tiles
-    assert tile(2, 64, 1300, 64, causal=True) == 32                       # ... but not where the tiles are dealt out
-    assert tile(4, 16, 2048, 64, causal=True) == 32                       # 128 pairs: half a round
+    assert tile(2, 64, 1300, 64, causal=True) == 16                       # ... and where the tiles are dealt out to a resident grid
+    assert tile(3, 12, 4096, 64, causal=True) == 32                       # 144 pairs: little more than half a round
+    assert tile(3, 20, 4096, 64, causal=True) == 16                       # 240 pairs: causal launches from 7/8 of a round on,
+    assert tile(5, 20, 4096, 64, causal=True) == 16                       # ... whatever the last round holds (400 pairs)
+    assert tile(5, 20, 2048, 64, causal=True) == 32                       # 200 pairs
     assert tile(4, 16, 4096, 64, has_mask=True) == 32                     # never with a mask
     assert tile(4, 32, 4096, 32) == 32 and tile(1, 32, 16384, 128) == 32  # head_dim 64 only
 

@@ -753,11 +753,15 @@ def test_kernel_with_16_row_matrix_tiles(gpu, B, R, L, dtype):
     (16, 16, 1000),     # ... with a ragged second tile
     (2, 85, 2500),      # five tiles per head: two pairs and the middle tile alone, ragged end
     (1, 16, 16384),     # 16 pairs per head, up to 32 key tiles below the diagonal
+    (2, 40, 4096),      # 320 pairs would be 1.25 rounds: tiles dealt out to a resident grid
+    (2, 64, 1300),      # ... three tiles per head, ragged end
+    (3, 20, 4096),      # 240 pairs: a single round, not quite full
 ])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_causal_kernel_with_16_row_matrix_tiles(gpu, B, R, L, dtype):
-    # Causal launches at head_dim 64 made of whole rounds of pairs of query tiles: the 16 x 16 kernel,
-    # whose waves own blocks of 16 queries dealt out so that all eight reach their diagonals together.
+    # Causal launches at head_dim 64 from seven eighths of a round of 512-query workgroups on (pairs of
+    # query tiles, or tiles dealt out to a resident grid): the 16 x 16 kernel, whose waves own blocks of
+    # 16 queries dealt out so that all eight reach their diagonals together.
     H = 64
     assert capi.launch_plan(B, R, L, H, causal=True)["matrix_tile"] == 16
     q, k, v = (_rand((B, L, R * H), 4050 + L + i).to(dtype) for i in range(3))
