@@ -806,6 +806,29 @@ def test_eight_wave_kernel_on_adversarial_scores(gpu, B, R, L, H, kind):
     assert scores.abs().max() > 20
 
 
+@pytest.mark.parametrize("B,R,L", [(4, 16, 4096), (16, 16, 1024), (2, 40, 4096)])
+@pytest.mark.parametrize("kind", ["std3", "rising", "falling"])
+def test_causal_16_row_kernel_on_adversarial_scores(gpu, B, R, L, kind):
+    # The same stress as above under the causal flag, where the 16 x 16 kernel leaves the blocks of a
+    # wave one after the other: the reference is overtaken inside the sub-tiles in which only some
+    # of a wave's blocks still take part (pairs of tiles, one pair per head, tiles dealt out).
+    H = 64
+    assert capi.launch_plan(B, R, L, H, causal=True)["matrix_tile"] == 16
+    q, k, v = (_rand((B, L, R * H), 4200 + L + i) for i in range(3))
+    if kind == "std3":
+        q, k = (q.float() * 3).half(), (k.float() * 3).half()
+    else:
+        g = torch.Generator().manual_seed(4207)
+        u = torch.randn(R * H, generator=g)
+        u = u / u.view(R, H).norm(dim=1).repeat_interleave(H)
+        ramp = torch.linspace(0, 1, L) if kind == "rising" else torch.linspace(1, 0, L)
+        q = (q.float() * 0.3 + 10.0 * u).half()
+        k = (k.float() * 0.3 + (10.0 * math.sqrt(H)) * ramp.view(1, L, 1) * u).half()
+    got = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, causal=True)
+    assert torch.isfinite(got.float()).all()
+    _check_pairs(got, q, k, v, H, [(0, 0), (B - 1, R // 2), (B - 1, R - 1)], mask=causal_mask(B, L))
+
+
 @pytest.mark.parametrize("B,R,L,H", [(2, 16, 4096, 64), (2, 64, 1024, 128)])
 @pytest.mark.parametrize("step_log2", [6.5, 14.0, 15.5, 16.5, 18.0, 21.0, 22.5, 26.0])
 def test_eight_wave_kernel_reference_lag(gpu, B, R, L, H, step_log2):
