@@ -199,32 +199,59 @@ hipError_t launch_pingpong(const fa::FwdParams& p, hipStream_t stream) {
     return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(NW * 64), args, lds, stream);
 }
 
-// The eight-wave kernel with its products written as 16 x 16 tiles (fwd_kernel_pp16), head_dim 64.
+// The eight-wave kernel with its products written as 16 x 16 tiles (fwd_kernel_pp16), head_dim 64
+// (64-row waves) and 128 (32-row waves).
 // Plain launches: on a full chip the clock follows the switching activity and the 16 x 16 x 32
-// instruction moves half as many accumulator registers per flop (measured, same box: 256
-// workgroups +2.9 and +3.6 %, 512 +3.5 %, 480 +1.1 %); where part of the chip idles the clock is not
-// held back and its 36 matrix instructions per sub-tile instead of 20 cost more than they save, and
-// a part-filled last round takes that from the whole launch (192 workgroups -5 to -9 %, 384 -3.4
-// and -4.6 %, 448 -0.7 %, 640 -1.0 %, 1152 -0.8 %): taken when the last round is at least seven
-// eighths full.  Causal launches in pairs of tiles: there the gain is the kernel's deal of 16-query
+// instruction moves half as many accumulator registers per flop; where part of the chip idles the
+// clock is not held back and its 36 (34) matrix instructions per sub-tile instead of 20 (18) cost
+// more than they save, and a part-filled last round takes that from the whole launch.  Measured on
+// the same box, by workgroups, head_dim 64: 256 +2.9 and +3.6 %, 480 +1.1 %, 512 +3.5 %; 192 -5 to
+// -9 %, 384 -3.4 and -4.6 %, 448 -0.7 %, 640 -1.0 %, 1152 -0.8 %.  head_dim 128: 224 +3.4 %, 256
+// +3.1 %, 480 +2.5 %, 512 +2.1 %, 1280 +3.1 %, 2048 +5.2 %; 192 -0.3 %, 384 -2.0 %, 448 +1.3 %, 640
+// -0.9 %, 800 -0.2 %, 1088 +0.1 %, 1600 -0.9 %.  Taken when the last round is at least seven
+// eighths full.
+// Causal launches in pairs of tiles or dealt out: there the gain is the kernel's deal of 16-query
 // blocks to the waves, which does not depend on the clock, and only an emptier single round loses
-// (144 pairs -4.3 %, 160 -6.2 %, 192 -1.4 and +1.3 %, 200 -0.6 %; 240 +3.6 %, 256 +5.5 %, 400
-// +1.4 %, 960 +4.5 and +7.5 %, 1152 +5.4 %): taken from seven eighths of a round on.
+// (head_dim 64: 144 pairs -4.3 %, 160 -6.2 %, 192 -1.4 and +1.3 %, 200 -0.6 %; 240 +3.6 %, 256
+// +5.5 %, 400 +1.4 %, 960 +4.5 and +7.5 %, 1152 +5.4 %, dealt +3.2 to +4.7 %; head_dim 128: 1024
+// pairs +5.1 and +5.4 %, dealt +4.2 %): taken from seven eighths of a round on.
 bool use_tiles16(int64_t H, Shape sh, const fa::FwdParams& p, bool causal) {
-    if (H != 64 || sh.waves != 8 || sh.nqb != 2) return false;
-    if (causal) return 8 * (int64_t)p.total_wgs >= 7 * kNumCu;     // (a dealt launch is a whole resident grid)
+    if (sh.waves != 8 || !((H == 64 && sh.nqb == 2) || H == 128)) return false;
+    if (8 * (int64_t)p.total_wgs < 7 * kNumCu) return false;
+    if (causal) return true;            // (a dealt launch is a whole resident grid)
+    if (H == 64 && p.total_wgs < kNumCu) return false;
     const int last = p.total_wgs % kNumCu;
-    return p.total_wgs >= kNumCu && (last == 0 || 8 * last >= 7 * kNumCu);
+    return last == 0 || 8 * last >= 7 * kNumCu;
 }
 
-template <bool BF, int MODE>
+template <int H, bool BF, int MODE>
 hipError_t launch_pp16(const fa::FwdParams& p, hipStream_t stream) {
-    constexpr int lds = fa::lds_bytes_pingpong<64, 2>();
-    auto kernel = BF ? fa::bf16::fwd_kernel_pp16<8, true, MODE> : fa::fwd_kernel_pp16<8, true, MODE>;
+    constexpr int lds = fa::lds_bytes_pingpong<H, 2>();
+    auto kernel = BF ? fa::bf16::fwd_kernel_pp16<H, 8, true, MODE> : fa::fwd_kernel_pp16<H, 8, true, MODE>;
+    if constexpr (lds > 64 * 1024) {
+        const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kernel), lds);
+        if (e != hipSuccess) return e;
+    }
     fa::FwdParams params = p;
     void* args[] = {&params};
     return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(p.wgs_per_xcd * fa::kNumXcd), dim3(8 * 64), args,
                            lds, stream);
+}
+
+template <int H, bool BF>
+hipError_t launch_pp16_mode(int mode, const fa::FwdParams& p, hipStream_t stream) {
+    switch (mode) {
+        case fa::kPlain: return launch_pp16<H, BF, fa::kPlain>(p, stream);
+        case fa::kCausal: return launch_pp16<H, BF, fa::kCausal>(p, stream);
+        case fa::kCausalDealt: return launch_pp16<H, BF, fa::kCausalDealt>(p, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_tiles16(int64_t H, int mode, bool bf16, const fa::FwdParams& p, hipStream_t stream) {
+    if (H == 64) return bf16 ? launch_pp16_mode<64, true>(mode, p, stream) : launch_pp16_mode<64, false>(mode, p, stream);
+    if (H == 128) return bf16 ? launch_pp16_mode<128, true>(mode, p, stream) : launch_pp16_mode<128, false>(mode, p, stream);
+    return hipErrorInvalidValue;
 }
 
 template <int H, int MODE, bool BF>
@@ -396,18 +423,14 @@ int fa_fwd_strided(const void* q, const void* k, const void* v, const void* mask
     if (rc != FA_OK) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e;
-    if (causal && use_tiles16(H, shape, p, true) && p.heads_per_xcd > 0)
-        e = bf16 ? launch_pp16<true, fa::kCausalDealt>(p, s) : launch_pp16<false, fa::kCausalDealt>(p, s);
-    else if (causal && use_tiles16(H, shape, p, true))
-        e = bf16 ? launch_pp16<true, fa::kCausal>(p, s) : launch_pp16<false, fa::kCausal>(p, s);
+    if (mask == nullptr && use_tiles16(H, shape, p, causal))
+        e = launch_tiles16(H, causal ? (p.heads_per_xcd > 0 ? fa::kCausalDealt : fa::kCausal) : fa::kPlain, bf16, p, s);
     else if (causal && p.heads_per_xcd > 0)
         e = dispatch<fa::kCausalDealt>(H, shape, p, s, bf16);
     else if (causal)
         e = dispatch<fa::kCausal>(H, shape, p, s, bf16);
     else if (mask != nullptr)
         e = dispatch<fa::kAdditive>(H, shape, p, s, bf16);
-    else if (use_tiles16(H, shape, p, false))
-        e = bf16 ? launch_pp16<true, fa::kPlain>(p, s) : launch_pp16<false, fa::kPlain>(p, s);
     else
         e = dispatch<fa::kPlain>(H, shape, p, s, bf16);
     return static_cast<int>(e);

@@ -112,9 +112,9 @@ int fa_fwd_strided(const void* q, const void* k, const void* v, const void* mask
  * pairs of query tiles per head for a causal launch of the eight-wave kernel and for those masked
  * launches of it that pairs cost no round of the chip; 0, or, when the
  * query tiles of a causal launch are dealt out to a resident grid, the heads per XCD; the edge of
- * the matrix instruction's tile, 32, or 16 at head_dim 64 for plain launches whose workgroups fill
- * whole rounds of the chip (the last round at least seven eighths full) and for causal launches in
- * pairs of tiles from seven eighths of a round on.
+ * the matrix instruction's tile, 32, or 16 at head_dim 64 and 128 for plain launches of the eight-wave
+ * kernel whose workgroups fill whole rounds of the chip (the last round at least seven eighths full)
+ * and for its causal launches from seven eighths of a round on.
  * The reference has no counterpart (its grid is fixed at (B, L / chunk_size, R),
  * reference include/fused_attn.cuh:872-883).
  */

@@ -221,7 +221,14 @@ def test_the_16_row_matrix_tile_is_taken_on_whole_rounds_only():
     assert tile(5, 20, 4096, 64, causal=True) == 16                       # ... whatever the last round holds (400 pairs)
     assert tile(5, 20, 2048, 64, causal=True) == 32                       # 200 pairs
     assert tile(4, 16, 4096, 64, has_mask=True) == 32                     # never with a mask
-    assert tile(4, 32, 4096, 32) == 32 and tile(1, 32, 16384, 128) == 32  # head_dim 64 only
+    assert tile(4, 32, 4096, 32) == 32 and tile(16, 16, 4096, 16) == 32   # head_dim 64 and 128 only
+    assert (wgs(1, 32, 16384, 128), tile(1, 32, 16384, 128)) == (2048, 16)    # c4: eight rounds of 256-query workgroups
+    assert (wgs(4, 40, 2048, 128), tile(4, 40, 2048, 128)) == (1280, 16)      # the reference's benchmark shape: five rounds
+    assert (wgs(1, 28, 2048, 128), tile(1, 28, 2048, 128)) == (224, 16)       # seven eighths of a round
+    assert (wgs(1, 48, 2048, 128), tile(1, 48, 2048, 128)) == (384, 32)       # one and a half rounds
+    assert (wgs(1, 24, 2048, 128), tile(1, 24, 2048, 128)) == (192, 32)
+    assert tile(1, 32, 16384, 128, causal=True) == 16 and tile(4, 40, 2048, 128, causal=True) == 16   # pairs; dealt
+    assert tile(4, 40, 2048, 128, has_mask=True) == 32
 
 
 def test_missing_library_fails_loudly(monkeypatch):

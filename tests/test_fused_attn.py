@@ -747,6 +747,40 @@ def test_kernel_with_16_row_matrix_tiles(gpu, B, R, L, dtype):
     assert torch.equal(same.permute(0, 2, 1, 3).reshape(B, L, R * H), got)
 
 
+@pytest.mark.parametrize("B,R,L,causal", [
+    (2, 64, 1024, False),    # 512 workgroups of 256 queries: two whole rounds
+    (4, 40, 2048, False),    # the reference's benchmark shape: five rounds
+    (4, 64, 1250, False),    # five tiles per head, ragged end (1280 workgroups)
+    (1, 28, 2048, False),    # a single round seven eighths full
+    (1, 8, 16384, False),    # 256 key tiles per workgroup
+    (2, 64, 1024, True),     # causal: two pairs per head
+    (1, 32, 16384, True),    # ... 32 pairs per head
+    (4, 64, 1250, True),     # ... five tiles per head, ragged end, dealt out to a resident grid
+    (5, 17, 1250, True),     # ... in pairs with the middle one alone
+    (2, 40, 2048, True),     # ... tiles dealt out to a resident grid
+])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_kernel_with_16_row_matrix_tiles_at_head_dim_128(gpu, B, R, L, causal, dtype):
+    # The 16 x 16 kernel with 32-row waves (two blocks of 16 queries, dealt w and 15 - w under the causal flag)
+    H = 128
+    assert capi.launch_plan(B, R, L, H, causal=causal)["matrix_tile"] == 16
+    q, k, v = (_rand((B, L, R * H), 4080 + L + i).to(dtype) for i in range(3))
+    got, lse = capi.forward(q.to(gpu), k.to(gpu), v.to(gpu), H, causal=causal, return_lse=True)
+    assert torch.isfinite(got.float()).all()
+    tol = TOL if dtype == torch.float16 else BF16_TOL
+    mask = causal_mask(1, L) if causal else None
+    for b, h in [(0, 0), (B // 2, R // 3), (B - 1, R - 1)]:
+        sl = slice(h * H, (h + 1) * H)
+        rows = slice(None) if L <= 4096 else torch.cat([torch.arange(0, 600), torch.arange(L - 600, L), torch.arange(600, L - 600, 97)])
+        want = attention(q[b:b + 1, :, sl], k[b:b + 1, :, sl], v[b:b + 1, :, sl], H, mask=mask)
+        assert (got[b, rows, sl].float().cpu() - want[0, rows]).abs().max().item() <= tol, (b, h)
+        want = attention_lse(q[b:b + 1, :, sl], k[b:b + 1, :, sl], H, mask=mask)[0, 0]
+        assert ((lse[b, h].cpu() - want).abs() / (1 + want.abs()))[rows].max().item() <= 1e-3, (b, h)
+    heads = lambda t: t.view(B, L, R, H).permute(0, 2, 1, 3).contiguous().to(gpu)
+    same = capi.forward(heads(q), heads(k), heads(v), H, layout="bhld", causal=causal)
+    assert torch.equal(same.permute(0, 2, 1, 3).reshape(B, L, R * H), got)
+
+
 @pytest.mark.parametrize("B,R,L", [
     (4, 16, 4096),      # 256 pairs of 512-query tiles
     (16, 16, 1024),     # one pair per head: both tiles are diagonal tiles
