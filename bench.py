@@ -34,13 +34,13 @@ PEAK_TFLOPS_FP16 = 2500.0   # MI355X dense fp16 MFMA, published
 # what the same counter reads for the 1 GiB calibration copy below: 2.000 for fetch, 1.000 for
 # write) and are quoted here with the file that holds the counter summary.  Workloads without a
 # counter run report null.  The counter runs were made at the commit that last touched each file's
-# counters (c3 425c6ed; c3_mask c1f4501; c4 and the projection 274d331; readme 4697fa4); the kernel
+# counters (c3 425c6ed; c3_mask c1f4501; c4 and readme at the commit that added the 16 x 16 kernel for head_dim 128; the projection 274d331); the kernel
 # each of these workloads runs has not changed since.
 MEASURED_TRAFFIC = {
     "c3": (134.4e6, "profiles/fwd_kernel_pp16_c3.md"),
     "c3_mask": (470.0e6, "profiles/fwd_kernel_pingpong_mask.md"),
-    "c4": (806.5e6, "profiles/fwd_kernel_pingpong_c4.md"),
-    "readme": (335.7e6, "profiles/fwd_kernel_pingpong_readme.md"),
+    "c4": (805.5e6, "profiles/fwd_kernel_pp16_c4.md"),
+    "readme": (335.7e6, "profiles/fwd_kernel_pp16_readme.md"),
     "qkv_proj_c3": (269.4e6, "profiles/qkv_proj_kernel_c3.md"),
     "qkv_proj_readme": (2181.4e6, "profiles/qkv_proj_kernel_readme.md"),
 }
