@@ -34,7 +34,7 @@ PEAK_TFLOPS_FP16 = 2500.0   # MI355X dense fp16 MFMA, published
 # what the same counter reads for the 1 GiB calibration copy below: 2.000 for fetch, 1.000 for
 # write) and are quoted here with the file that holds the counter summary.  Workloads without a
 # counter run report null.  The counter runs were made at the commit that last touched each file's
-# counters (c3 425c6ed; c3_mask c1f4501; c4 and readme at the commit that added the 16 x 16 kernel for head_dim 128; the projection 274d331); the kernel
+# counters (c3, c4 and readme at the commit that gave the 16 x 16 kernel its conflict-free K chunk order; c3_mask c1f4501; the projection 274d331); the kernel
 # each of these workloads runs has not changed since.
 MEASURED_TRAFFIC = {
     "c3": (134.4e6, "profiles/fwd_kernel_pp16_c3.md"),
