@@ -219,7 +219,7 @@ bool use_tiles16(int64_t H, Shape sh, const fa::FwdParams& p, bool causal) {
     if (sh.waves != 8 || !((H == 64 && sh.nqb == 2) || H == 128)) return false;
     if (8 * (int64_t)p.total_wgs < 7 * kNumCu) return false;
     if (causal) return true;            // (a dealt launch is a whole resident grid)
-    if (H == 64 && p.total_wgs < kNumCu) return false;
+    if (H == 64 && p.total_wgs < kNumCu) return false;     // (224 and 240 workgroups: +1.6 and +2.5 % at L = 4096, -1.4 % at L = 1024)
     const int last = p.total_wgs % kNumCu;
     return last == 0 || 8 * last >= 7 * kNumCu;
 }
