@@ -34,15 +34,15 @@ PEAK_TFLOPS_FP16 = 2500.0   # MI355X dense fp16 MFMA, published
 # what the same counter reads for the 1 GiB calibration copy below: 2.000 for fetch, 1.000 for
 # write) and are quoted here with the file that holds the counter summary.  Workloads without a
 # counter run report null.  The counter runs were made at the commit that last touched each file's
-# counters (c3, c4 and readme at the commit that gave the 16 x 16 kernel its conflict-free K chunk order; c3_mask c1f4501; the projection 274d331); the kernel
+# counters (c3, c4 and readme at the commit that gave the 16 x 16 kernel its conflict-free K chunk order; c3_mask c1f4501; the projection at the commit that rewrote it on 16 x 16 x 32 instructions); the kernel
 # each of these workloads runs has not changed since.
 MEASURED_TRAFFIC = {
     "c3": (134.4e6, "profiles/fwd_kernel_pp16_c3.md"),
     "c3_mask": (470.0e6, "profiles/fwd_kernel_pingpong_mask.md"),
     "c4": (805.5e6, "profiles/fwd_kernel_pp16_c4.md"),
     "readme": (335.7e6, "profiles/fwd_kernel_pp16_readme.md"),
-    "qkv_proj_c3": (269.4e6, "profiles/qkv_proj_kernel_c3.md"),
-    "qkv_proj_readme": (2181.4e6, "profiles/qkv_proj_kernel_readme.md"),
+    "qkv_proj_c3": (268.6e6, "profiles/qkv_proj_kernel_c3.md"),
+    "qkv_proj_readme": (2181.2e6, "profiles/qkv_proj_kernel_readme.md"),
 }
 
 # Launches made before the counted warm-up until this much time has passed: the chip needs a few
