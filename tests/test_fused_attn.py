@@ -400,30 +400,37 @@ def test_heads_and_batches_are_independent_bitwise(gpu):
     assert not torch.equal(out[0, :, H:2 * H], base[0, :, H:2 * H])
 
 
-def test_launch_can_be_captured_in_a_graph_and_replayed(gpu):
+@pytest.mark.parametrize("B,R,L,H,causal", [
+    (2, 16, 1024, 64, False),       # the four-wave kernel
+    (4, 16, 2048, 64, False),       # the 16 x 16 kernel, one whole round
+    (2, 64, 1024, 128, False),      # ... at head_dim 128
+    (16, 16, 1024, 64, True),       # ... causal, a pair of tiles per workgroup
+    (2, 40, 2048, 128, True),       # ... causal, tiles dealt out to a resident grid
+])
+def test_launch_can_be_captured_in_a_graph_and_replayed(gpu, B, R, L, H, causal):
     # The library allocates nothing and clears nothing at launch time, so a launch on a capturing
     # stream is recorded as a single kernel node.  Replays must follow the contents of the (static)
     # input buffers and agree bitwise with eager launches, with eager work between the replays.
     import fused_attn
 
-    B, R, L, H = 2, 16, 1024, 64
+    forward = lambda a, b_, c: fused_attn.attention_forward_ex(a, b_, c, H, causal=causal)
     q, k, v = (_rand((B, L, R * H), 2400 + i).to(gpu) for i in range(3))
-    eager0 = fused_attn.attention_forward(H, 64, q, k, v)        # also the warm-up launch
+    eager0 = forward(q, k, v)        # also the warm-up launch
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        out = fused_attn.attention_forward(H, 64, q, k, v)
+        out = forward(q, k, v)
     for rep in range(4):
         if rep:
             q.copy_(_rand((B, L, R * H), 2410 + rep))            # new inputs in the captured buffers
-        eager = fused_attn.attention_forward(H, 64, q, k, v)
+        eager = forward(q, k, v)
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
         if rep == 0:
             assert torch.equal(out, eager0)
-    want = attention(q.cpu(), k.cpu(), v.cpu(), H)
-    assert _max_err(out, want) <= TOL
+    pairs = [(0, 0), (B - 1, R // 2), (B - 1, R - 1)]
+    _check_pairs(out, q.cpu(), k.cpu(), v.cpu(), H, pairs, mask=causal_mask(B, L) if causal else None)
 
 
 def _random_cases(n, seed):
